@@ -13,9 +13,6 @@
 //     ds_write), one SGPR offset per piece, so the only VGPR per piece is a constant per-lane
 //     row offset;  the register-staged form of this tile (csrc/experimental/gemm_rs.hip) lost
 //     on its 16 ds_write_b128 per K-tile (PERF.md "Round 3: the 256x256 feed");
-//   * the disassembly of hipBLASLt's own MT256x256x64 kernel on this image (the library the
-//     table used to pick for these shapes) has exactly these resources: 256 threads, 256
-//     AGPR accumulators, 16x16x32 MFMAs, LDS-DMA loads -- the schedule below is our own.
 //
 // Schedule (one K-tile t; LDS = a ring of five 32-KiB slots, tile t's X and W halves in slots
 // 2t and 2t+1 mod 5; every index static):
