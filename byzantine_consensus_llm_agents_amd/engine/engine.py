@@ -55,7 +55,8 @@ import torch
 
 from ..bcg.config import ENGINE_CONFIG
 from ..models.config import ModelConfig, get_model_config
-from ..models.transformer import AttnMeta, DecoderModel, TPGroup
+from ..models import build_model
+from ..models.transformer import AttnMeta, TPGroup
 from ..ops import get_ops
 from ..utils.trace import PhaseTimer
 from .guided.compiler import FSMRegistry
@@ -89,6 +90,7 @@ class EngineArgs:
     prefix_caching: bool = True
     use_hip_graphs: bool = True
     kv_cache_gb: Optional[float] = None
+    kv_pool_tokens: Optional[int] = None  # size the KV pool for exactly this many tokens (rounded up to blocks)
     honor_max_num_seqs: bool = False
     dtype: torch.dtype = torch.bfloat16
     device: Optional[str] = None
@@ -196,10 +198,14 @@ class InferenceEngine:
         self.ops = get_ops(self.backend)
 
         model_dir = args.weights if args.weights not in ("random", "auto") else None
-        self.tokenizer = load_tokenizer(args.model, model_dir)
+        if model_dir and not os.path.exists(os.path.join(model_dir, "tokenizer.json")) and cfg.family == "mofidra":
+            from .tokenizer import IdTokenizer
+            self.tokenizer = IdTokenizer(cfg.vocab_size)  # a checkpoint of weights only: prompts are token ids
+        else:
+            self.tokenizer = load_tokenizer(args.model, model_dir)
         if self.tokenizer.vocab_size > cfg.vocab_size:
             raise ValueError("tokenizer larger than the model vocabulary")
-        self.model = DecoderModel(cfg, self.ops, self.device, args.dtype, self.tp, quant=args.quantization)
+        self.model = build_model(cfg, self.ops, self.device, args.dtype, self.tp, quant=args.quantization)
         with self.timer.phase("load_weights"):
             if model_dir:
                 from ..models.loader import load_safetensors_dir
@@ -277,7 +283,7 @@ class InferenceEngine:
         a, m = self.args, self.model
         bs = a.kv_block_size
         kv_dtype = self.kv_dtype()
-        per_block = 2 * m.cfg.num_layers * m.n_kv * bs * m.hd * torch.tensor([], dtype=kv_dtype).element_size()
+        per_block = m.kv_block_bytes(bs, kv_dtype)
         want_tokens = a.max_batch_seqs * a.max_model_len
         if a.kv_cache_gb:
             budget = int(a.kv_cache_gb * 2 ** 30)
@@ -294,21 +300,20 @@ class InferenceEngine:
         else:
             budget = 256 * 2 ** 20
         num_blocks = max(16, min(budget // per_block, want_tokens // bs + 1))
-        self.k_cache = torch.zeros((m.cfg.num_layers, num_blocks, m.n_kv, bs, m.hd), dtype=kv_dtype,
-                                   device=self.device)
-        # V is stored transposed per block-head (see ops/reference.py)
-        self.v_cache = torch.zeros((m.cfg.num_layers, num_blocks, m.n_kv, m.hd, bs), dtype=kv_dtype,
-                                   device=self.device)
+        if a.kv_pool_tokens:
+            num_blocks = (a.kv_pool_tokens + bs - 1) // bs + 1  # + the scratch block
+        # the model lays out its own cache (one tensor over all layers, or one per layer run)
+        self.k_cache, self.v_cache = m.alloc_kv(num_blocks, bs, kv_dtype, self.device)
         from ..runtime import BlockManager
         # block 0 is scratch (padding rows of graph buckets write there); never handed out
         self.blocks = BlockManager(num_blocks - 1, bs)
         self.num_blocks = num_blocks
         self.max_blocks_per_seq = (a.max_model_len + bs - 1) // bs
-        self.kv_bytes = 2 * self.k_cache.numel() * self.k_cache.element_size()
+        self.kv_bytes = num_blocks * per_block
 
     def _decode_ws_bytes(self) -> int:
-        if not hasattr(self.ops, "decode_workspace_numel"):
-            return 0
+        if not hasattr(self.ops, "decode_workspace_numel") or not getattr(self.model, "supports_cascade", True):
+            return 0  # (models with their own decode attention size its scratch per launch)
         from .graphs import MAX_ROWS
         a, m = self.args, self.model
         rows = min(MAX_ROWS, max(a.max_batch_seqs, 1))
@@ -363,13 +368,16 @@ class InferenceEngine:
         ws = self._decode_ws_bytes() // 4
         self.decode_ws = torch.empty(ws, dtype=torch.float32, device=dev) if ws else None
         self.cascade = None
-        if self.backend == "hip" and self.args.cascade_decode and os.environ.get("BCG_CASCADE", "1") != "0":
+        if (self.backend == "hip" and self.args.cascade_decode and os.environ.get("BCG_CASCADE", "1") != "0"
+                and getattr(self.model, "supports_cascade", True)):
             from .cascade import CascadeTables
             self.cascade = CascadeTables(cap, dev, self.args.kv_block_size)
         self._layout_dirty = True  # live rows changed since the cascade tables were built
         rows_fn = getattr(self.ops, "prefill_tile_rows", None)
         self._tile_rows = (rows_fn(self.model.hd, self.kv_dtype() == torch.float8_e4m3fn, self.max_blocks_per_seq)
                            if rows_fn else 64)
+        self._tile_rows = getattr(self.model, "prefill_tile_rows", self._tile_rows)
+        self._streams: Dict[str, "_Request"] = {}  # open token streams (stream_step), by caller id
 
     def _phys(self, blocks: List[int]) -> List[int]:
         return [b + 1 for b in blocks]  # manager ids are shifted past scratch block 0
@@ -396,6 +404,83 @@ class InferenceEngine:
             if r.exc is not None:
                 raise r.exc
         return [r.text for r in reqs]
+
+    def generate_ids(self, prompts: List[List[int]], max_tokens, temperature=0.0) -> List[List[int]]:
+        """`generate` for callers that hold token ids (a checkpoint without a tokenizer, offline
+        scoring): the same admission, paged prefill, decode bursts and sampler; unguided.
+        ``max_tokens`` / ``temperature``: one value or one per prompt.  Returns the generated ids."""
+        if not self.is_driver:
+            raise RuntimeError("generate_ids() on a TP follower")
+        n = len(prompts)
+        mt = list(max_tokens) if isinstance(max_tokens, (list, tuple)) else [max_tokens] * n
+        tp = list(temperature) if isinstance(temperature, (list, tuple)) else [temperature] * n
+        reqs = [self._make_request(list(p), m, t, None) for p, m, t in zip(prompts, mt, tp)]
+        with self._cv:
+            self.stats["calls"] += 1
+            self._incoming.extend(r for r in reqs if not r.event.is_set())
+            self._cv.notify_all()
+        if self.async_mode:
+            for r in reqs:
+                r.event.wait()
+        else:
+            with self._device_ctx():
+                while not all(r.event.is_set() for r in reqs):
+                    self._iterate()
+        for r in reqs:
+            if r.exc is not None:
+                raise r.exc
+        return [list(r.token_ids) for r in reqs]
+
+    # ---- token streams: the caller supplies every token (scoring, trace replay) ----
+    def stream_step(self, entries, end=()) -> torch.Tensor:
+        """One engine step over caller-supplied tokens.  ``entries``: [(stream id, tokens, want)]
+        -- the next tokens of each stream (a stream opens at its first entry: a state row and,
+        as it grows, KV blocks from the engine's pool) and the offsets among them whose logits
+        are wanted.  All entries run as ONE packed batch through the model's forward (prompt
+        portions through the prefill tiles, one-token entries through the decode kernel when the
+        model splits them).  ``end``: streams to close after the step (row and blocks are given
+        back).  Returns fp32 logits [sum of wants, vocab] in entry order."""
+        bs = self.args.kv_block_size
+        wave, chunk, want = [], [], []
+        with self._device_ctx():
+            for sid, tokens, w in entries:
+                req = self._streams.get(sid)
+                if req is None:
+                    free = [i for i, r in enumerate(self.slots) if r is None]
+                    if not free:
+                        raise RuntimeError("no free state row for a new stream")
+                    req = _Request(_Seq(0, [], 0, 0.0, None))
+                    req.row, req.pending = free[0], True
+                    self.slots[req.row] = self._streams[sid] = req
+                seq = req.seq
+                a = len(seq.prompt_ids)
+                if not tokens or a + len(tokens) > self.args.max_model_len:
+                    raise ValueError("stream entry empty or beyond max_model_len")
+                need = (a + len(tokens) + bs - 1) // bs - len(seq.blocks)
+                if need > 0:
+                    more = self.blocks.grow(need)
+                    if not more:
+                        raise RuntimeError("KV pool exhausted")
+                    seq.blocks.extend(more)
+                seq.prompt_ids.extend(int(t) for t in tokens)
+                chunk.append((len(wave), a, a + len(tokens)))
+                wave.append(seq)
+                want.append(list(w))
+            logits = None
+            if chunk:
+                table_cpu = self._block_table(wave, len(wave))
+                tokens, meta, _, n_want = self._plan_chunk(wave, chunk, table_cpu, want=want)
+                if not n_want:
+                    meta.logits_idx = meta.logits_idx[:1]
+                logits = self.model.forward(tokens, meta, self.k_cache, self.v_cache)[:n_want].float()
+                for (r, _, b) in chunk:
+                    wave[r].done_pos = b
+            for sid in end:
+                req = self._streams.pop(sid, None)
+                if req is not None:
+                    self.blocks.free(req.seq.blocks)
+                    self.slots[req.row] = None
+        return logits
 
     def _make_request(self, p_ids: List[int], max_tokens: int, temperature: float,
                       fsm_key: Optional[str]) -> "_Request":
@@ -825,6 +910,7 @@ class InferenceEngine:
                     toks = toks[:-1]
                 self.stats["generated_tokens"] += counts[i]
                 text = self.tokenizer.decode_bytes(toks).decode("utf-8", errors="replace")
+                req.token_ids = toks
                 self.blocks.free(req.seq.blocks)
                 self.slots[i] = None
                 req.finish(text)
@@ -916,7 +1002,10 @@ class InferenceEngine:
         self.stats["prefill_full_chunks"] += len(plans) - (1 if chunk and not hold_tail else 0)
         return plans
 
-    def _plan_chunk(self, wave, chunk, table_cpu):
+    def _plan_chunk(self, wave, chunk, table_cpu, want=None):
+        """Device metadata of one packed step over the segments ``chunk`` = [(wave index, first
+        position, end position)].  Logits rows: the last token of every prompt that ends in the
+        chunk, or -- ``want``: per segment, offsets into it -- exactly the rows asked for."""
         bs = self.args.kv_block_size
         toks, pos, slots, q_start, seq_lens, rows, last_idx, last_rows = [], [], [], [0], [], [], [], []
         for r, a, b in chunk:
@@ -929,19 +1018,26 @@ class InferenceEngine:
             q_start.append(q_start[-1] + (b - a))
             seq_lens.append(b)
             rows.append(r)
-            if b == len(s.prompt_ids):
+            if want is not None:
+                last_idx.extend(q_start[-2] + o for o in want[len(rows) - 1])
+            elif b == len(s.prompt_ids):
                 last_idx.append(q_start[-1] - 1)
                 last_rows.append(r)
         # query tiles for the HIP prefill kernel (ops.prefill_tile_rows rows), deepest (most keys) first
         tr = self._tile_rows
-        tiles = []
+        tiles, single = [], []
+        split = getattr(self.model, "split_single_rows", False)
         for i, (r, a, b) in enumerate(chunk):
+            if split and b - a == 1:  # a decoded token beside prompt portions: the decode kernel's
+                single.append((q_start[i], i))
+                continue
             for t in range(q_start[i], q_start[i + 1], tr):
                 tiles.append((b - (q_start[i + 1] - t), i, t, min(t + tr, q_start[i + 1])))
         tiles.sort(key=lambda x: -x[0])
         i32 = torch.int32
         meta = AttnMeta(
-            tiles=self._h2d(torch.tensor([x[1:] for x in tiles], dtype=i32)),
+            tiles=self._h2d(torch.tensor([x[1:] for x in tiles], dtype=i32).reshape(-1, 3)),
+            single=self._h2d(torch.tensor(single, dtype=i32).reshape(-1, 2)) if split else None,
             positions=self._h2d(torch.cat(pos).to(i32)),
             slots=self._h2d(torch.cat(slots).to(i32)),
             block_tables=self._h2d(table_cpu[rows]),
@@ -953,11 +1049,12 @@ class InferenceEngine:
             logits_idx=self._h2d(torch.tensor(last_idx if last_idx else [0], dtype=torch.int64)))
         tokens = self._h2d(torch.tensor(toks, dtype=i32))
         dest = self._h2d(torch.tensor(last_rows, dtype=torch.int64)) if last_rows else None
-        return tokens, meta, dest, len(last_rows)
+        return tokens, meta, dest, len(last_idx) if want is not None else len(last_rows)
 
     def _run_prefill(self, plans, n_rows: int) -> torch.Tensor:
         """Chunked packed prefill; returns last-token logits ``[n_rows, V]``."""
-        logits_out = torch.empty(n_rows, self.model.cfg.vocab_size, dtype=self.args.dtype, device=self.device)
+        logits_out = torch.empty(n_rows, self.model.cfg.vocab_size, device=self.device,
+                                 dtype=getattr(self.model, "logits_dtype", None) or self.args.dtype)
         for tokens, meta, dest, n_last in plans:
             logits = self.model.forward(tokens, meta, self.k_cache, self.v_cache)
             if n_last:
@@ -967,6 +1064,8 @@ class InferenceEngine:
 
     # -------------------------------------------------------------- decode
     def _sample(self, logits: torch.Tensor, st: Dict[str, torch.Tensor]):
+        if self.backend == "hip" and logits.dtype != torch.bfloat16:
+            logits = logits.to(torch.bfloat16)  # the guided sampler reads bf16 rows
         self.ops.sample_step(logits, self.fsm.table, self.fsm.dist, st["fsm_base"], st["fsm_state"],
                              st["gen_count"], st["max_new"], st["temperature"], st["row_keys"],
                              st["done"], st["seq_lens"], st["out_tokens"], st["next_tokens"],
@@ -1011,12 +1110,13 @@ class InferenceEngine:
 
 
 class _Request:
-    __slots__ = ("seq", "row", "text", "exc", "event", "pending", "enq_burst", "limit")
+    __slots__ = ("seq", "row", "text", "exc", "event", "pending", "enq_burst", "limit", "token_ids")
 
     def __init__(self, seq: _Seq, enq_burst: int = 0):
         self.seq, self.row, self.text, self.exc, self.pending = seq, -1, "", None, False
         self.enq_burst = enq_burst
         self.limit = None  # the stats counter of a context-limited request
+        self.token_ids: List[int] = []  # the generated tokens (set when the request is reaped)
         self.event = threading.Event()
 
     def finish(self, text: str):

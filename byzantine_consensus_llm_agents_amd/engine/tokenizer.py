@@ -177,6 +177,42 @@ class BCGTokenizer:
         return [self.token_bytes(i) for i in range(self.vocab_size)]
 
 
+class IdTokenizer:
+    """Tokenizer of a checkpoint that ships none: token i is the text ``"i "`` (prompts are
+    whitespace-separated token ids).  No end-of-sequence token: a request ends at its
+    ``max_tokens``.  Same surface as `BCGTokenizer`."""
+
+    synthetic, name = True, "token-ids"
+
+    def __init__(self, vocab_size: int):
+        self.vocab_size = vocab_size
+        self.eos_token_ids, self.eos_token_id, self.special_ids = [-1], None, set()
+
+    def encode(self, text: str) -> List[int]:
+        ids = [int(t) for t in text.split()]
+        if any(not 0 <= i < self.vocab_size for i in ids):
+            raise ValueError("token id outside the vocabulary")
+        return ids
+
+    def encode_batch(self, texts: List[str]) -> List[List[int]]:
+        return [self.encode(t) for t in texts]
+
+    def encode_batch_safe(self, texts: List[str]):
+        return self.encode_batch(texts), 0
+
+    def token_bytes(self, i: int) -> bytes:
+        return f"{i} ".encode()
+
+    def decode_bytes(self, ids: List[int]) -> bytes:
+        return b"".join(self.token_bytes(i) for i in ids)
+
+    def decode(self, ids: List[int]) -> str:
+        return self.decode_bytes(ids).decode()
+
+    def all_token_bytes(self) -> List[bytes]:
+        return [self.token_bytes(i) for i in range(self.vocab_size)]
+
+
 def encodable(text: str) -> str:
     """`text` with every lone surrogate replaced by U+FFFD (the same object when it has none)."""
     try:

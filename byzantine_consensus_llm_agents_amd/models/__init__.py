@@ -1,0 +1,14 @@
+"""Model registry: configuration family -> model class."""
+
+
+def model_class(family: str):
+    if family == "mofidra":
+        from .mofidra import MofidraModel
+        return MofidraModel
+    from .transformer import DecoderModel
+    return DecoderModel
+
+
+def build_model(cfg, ops, device, dtype, tp=None, quant=None):
+    """The model class that serves ``cfg`` (chosen by ``cfg.family``)."""
+    return model_class(cfg.family)(cfg, ops, device, dtype, tp, quant=quant)

@@ -60,6 +60,152 @@ class ModelConfig:
         return asdict(self)
 
 
+@dataclass(frozen=True)
+class MixerSpec:
+    """One differential-attention mixer: ``heads`` query heads over ``kv_heads`` key/value
+    heads, ``maps`` softmax maps per head (each with its own ``dim``-wide q/k slice, all over
+    the same ``vdim``-wide values), rotary on the first ``rot_dims`` features of every map."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    diff: float
+    rot_dims: int
+    rot_base: float
+    maps: int = 2
+
+    @property
+    def q_width(self) -> int:
+        return self.heads * self.maps * self.dim
+
+    @property
+    def k_width(self) -> int:
+        return self.kv_heads * self.maps * self.dim
+
+    @property
+    def v_width(self) -> int:
+        return self.kv_heads * self.vdim
+
+
+@dataclass(frozen=True)
+class FeedForwardSpec:
+    """kind "dense": one ``ff``-wide layer.  kind "moe": ``experts`` layers of width ``ff`` of
+    which a token uses ``top``, plus an always-on gated expert of width ``shared_ff`` (0 = none)."""
+    kind: str
+    ff: int
+    experts: int = 0
+    top: int = 0
+    shared_ff: int = 0
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    type: str
+    mixer: MixerSpec
+    mlp: Optional[FeedForwardSpec]
+
+
+@dataclass(frozen=True)
+class MofidraConfig:
+    """Mofidra: parallel-sublayer decoder (one norm feeds the mixer and the feed-forward),
+    differential attention, dense or mixture-of-experts feed-forwards, a weight-shared loop
+    over a span of layers.  Everything is read from the model directory's config.json; the
+    attributes the engine asks every model for (sizes, ``num_layers`` = cache-holding layer
+    runs) are derived."""
+    name: str
+    hidden_size: int
+    vocab_size: int
+    layers: tuple
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    rms_eps: float = 1e-6
+    embed_scale: float = 1.0
+    family: str = "mofidra"
+    max_position: int = 1 << 20
+    tie_embeddings: bool = False
+
+    @classmethod
+    def from_dict(cls, c: dict, name: str = "mofidra") -> "MofidraConfig":
+        layers = []
+        for entry in c["layers"]:
+            if entry["type"] != "attention":
+                raise ValueError(f"Mofidra: unknown mixer type {entry['type']!r}")
+            m = entry["mixer"]
+            rot = m.get("rot") or {"dims": 0, "base": 10000.0}
+            mixer = MixerSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]),
+                              vdim=int(m["vdim"]), scale=float(m["scale"]), diff=float(m["diff"]),
+                              rot_dims=int(rot["dims"]), rot_base=float(rot["base"]))
+            if mixer.heads % mixer.kv_heads or mixer.rot_dims % 2 or mixer.rot_dims > mixer.dim:
+                raise ValueError("Mofidra: heads must be a multiple of kv_heads, rot.dims even and <= dim")
+            f = entry.get("mlp")
+            mlp = None
+            if f is not None and f["kind"] == "dense":
+                mlp = FeedForwardSpec("dense", int(f["ff"]))
+            elif f is not None and f["kind"] == "moe":
+                shared = f.get("shared") or {}
+                mlp = FeedForwardSpec("moe", int(f["expert"]["ff"]), int(f["router"]["experts"]),
+                                      int(f["router"]["top"]), int(shared.get("ff", 0)))
+                if not 1 <= mlp.top <= mlp.experts:
+                    raise ValueError("Mofidra: router.top must be in [1, experts]")
+            elif f is not None:
+                raise ValueError(f"Mofidra: unknown feed-forward kind {f['kind']!r}")
+            layers.append(LayerSpec(entry["type"], mixer, mlp))
+        loop = c.get("loop") or {}
+        start, stop = int(loop.get("start", 0)), int(loop.get("stop", 0))
+        times = int(loop.get("times", 1))
+        if not 0 <= start <= max(start, stop) <= len(layers) or times < 1:
+            raise ValueError("Mofidra: loop span outside the layer list")
+        return cls(name=name, hidden_size=int(c["width"]), vocab_size=int(c["vocab"]), layers=tuple(layers),
+                   loop_start=start, loop_stop=max(start, stop), loop_times=times,
+                   rms_eps=float(c["norm"]["eps"]), embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)))
+
+    def to_dict(self) -> dict:
+        """The config.json form (inverse of `from_dict`)."""
+        out = []
+        for l in self.layers:
+            m = l.mixer
+            entry = {"type": l.type, "mixer": {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim, "vdim": m.vdim,
+                                               "scale": m.scale, "diff": m.diff,
+                                               "rot": {"dims": m.rot_dims, "base": m.rot_base}}, "mlp": None}
+            if l.mlp is not None and l.mlp.kind == "dense":
+                entry["mlp"] = {"kind": "dense", "ff": l.mlp.ff}
+            elif l.mlp is not None:
+                entry["mlp"] = {"kind": "moe", "expert": {"ff": l.mlp.ff},
+                                "router": {"experts": l.mlp.experts, "top": l.mlp.top}}
+                if l.mlp.shared_ff:
+                    entry["mlp"]["shared"] = {"ff": l.mlp.shared_ff}
+            out.append(entry)
+        return {"architecture": "Mofidra", "width": self.hidden_size, "vocab": self.vocab_size,
+                "embedding": {"scale": self.embed_scale}, "norm": {"eps": self.rms_eps}, "layers": out,
+                "loop": {"start": self.loop_start, "stop": self.loop_stop, "times": self.loop_times}}
+
+    @property
+    def layer_runs(self) -> tuple:
+        """Layer index of every layer run, in execution order: the loop span repeats
+        ``loop_times`` times with the same weights; every run keeps a KV cache of its own."""
+        n = len(self.layers)
+        span = tuple(range(self.loop_start, self.loop_stop))
+        return tuple(range(self.loop_start)) + span * self.loop_times + tuple(range(self.loop_stop, n))
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layer_runs)
+
+    def num_params(self) -> int:
+        W, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size + self.hidden_size
+        for l in self.layers:
+            m = l.mixer
+            n += W * (m.q_width + m.k_width + m.v_width) + W * m.heads * m.vdim + W + 4 * m.dim
+            f = l.mlp
+            if f is not None and f.kind == "dense":
+                n += 2 * W * f.ff
+            elif f is not None:
+                n += f.experts * (2 * W * f.ff + W + 1) + (2 * W * f.shared_ff + W if f.shared_ff else 0)
+        return n
+
+
 PRESETS = {
     "Qwen/Qwen3-8B": ModelConfig("Qwen/Qwen3-8B", "qwen3", 4096, 36, 32, 8, 128, 12288, 151936,
                                  qk_norm=True, max_position=40960),
@@ -90,9 +236,11 @@ ALIASES = {
 }
 
 
-def from_hf_config(path: str, name: Optional[str] = None) -> ModelConfig:
+def from_hf_config(path: str, name: Optional[str] = None):
     with open(os.path.join(path, "config.json")) as fh:
         c = json.load(fh)
+    if str(c.get("architecture", "")).lower() == "mofidra":
+        return MofidraConfig.from_dict(c, name or path)
     arch = (c.get("model_type") or "").lower()
     family = "qwen3" if arch == "qwen3" else ("qwen2" if arch == "qwen2" else "mistral")
     heads = c["num_attention_heads"]

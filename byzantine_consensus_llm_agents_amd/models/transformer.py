@@ -45,6 +45,9 @@ class AttnMeta:
     # that already finished (they idle in the batch until the host reaps them) one token, so
     # their KV is not streamed again every step; their outputs are ignored by the sampler
     attn_seq_lens: Optional[torch.Tensor] = None
+    # packed steps of models with `split_single_rows`: [n, 2] int32 {token row, sequence} of the
+    # one-token segments (a decoded token beside prompt portions); `tiles` then hold the others
+    single: Optional[torch.Tensor] = None
 
 
 class TPGroup:
@@ -121,6 +124,8 @@ class TPGroup:
 
 class DecoderModel:
     PROJECTIONS = ("qkv", "o", "gate_up", "down")
+    split_single_rows = False   # every segment of a packed step goes through the prefill tiles
+    supports_cascade = True     # shared-prefix decode attention (engine/cascade.py)
 
     def __init__(self, cfg: ModelConfig, ops, device, dtype=torch.bfloat16,
                  tp: Optional[TPGroup] = None, quant: Optional[str] = None):
@@ -146,6 +151,19 @@ class DecoderModel:
         self.lm_head: Optional[torch.Tensor] = None
         self.final_norm: Optional[torch.Tensor] = None
         self.cos_sin = None
+
+    # ------------------------------------------------------------- KV cache
+    def kv_block_bytes(self, block_size: int, dtype) -> int:
+        """Bytes of one KV block over all layers (K and V)."""
+        return 2 * self.cfg.num_layers * self.n_kv * block_size * self.hd * torch.tensor([], dtype=dtype).element_size()
+
+    def alloc_kv(self, num_blocks: int, block_size: int, dtype, device=None):
+        """(K [L, NB, n_kv, BS, hd], V [L, NB, n_kv, hd, BS]): V is stored transposed per
+        block-head (see ops/reference.py)."""
+        dev = device or self.device
+        L = self.cfg.num_layers
+        return (torch.zeros((L, num_blocks, self.n_kv, block_size, self.hd), dtype=dtype, device=dev),
+                torch.zeros((L, num_blocks, self.n_kv, self.hd, block_size), dtype=dtype, device=dev))
 
     # ------------------------------------------------------------- weights
     def _shapes(self):

@@ -23,8 +23,25 @@ def _torch_ops() -> SimpleNamespace:
                 tile_rows=64):
         return _ref.paged_attention(q, k_cache, v_cache, layer, block_tables, q_start, seq_lens, scale)
 
+    def multimap_attention(q, k_cache, v_cache, meta, scale, maps, lam, head_eps, out_scale, vdim):
+        # tiles / single-row lists only tell the HIP kernels how to walk the batch
+        q_start = meta.q_start
+        if q_start is None:  # decode: one row per sequence
+            q_start = torch.arange(q.shape[0] + 1, dtype=torch.int32, device=q.device)
+        lens = meta.seq_lens if meta.attn_seq_lens is None else meta.attn_seq_lens
+        return _ref.multimap_attention(q, k_cache, v_cache, meta.block_tables, q_start, lens, scale, maps,
+                                       lam, head_eps, out_scale, vdim)
+
     return SimpleNamespace(
         name="torch",
+        rmsnorm32=_ref.rmsnorm32,
+        embed_scale_rmsnorm=_ref.embed_scale_rmsnorm,
+        residual_add_rmsnorm32=_ref.residual_add_rmsnorm32,
+        rope_multi_kv_write=_ref.rope_multi_kv_write,
+        multimap_attention=multimap_attention,
+        act_fn=_ref.act_fn,
+        moe_route=_ref.moe_route,
+        moe_experts=_ref.moe_experts,
         linear=torch.nn.functional.linear,
         rmsnorm=_ref.rmsnorm,
         add_rmsnorm=_ref.add_rmsnorm,

@@ -332,3 +332,151 @@ def linear_fp8(xq, xs, wq, ws, bias=None, out_dtype=torch.bfloat16):
     if bias is not None:
         y = y + bias.float()
     return y.to(out_dtype)
+
+
+# ------------------------------------------------------------------ fp32 residual stream, multi-map attention, MoE
+# Mechanisms of the parallel-sublayer / differential-attention / mixture-of-experts decoders
+# (models/mofidra.py).  Conventions shared with csrc/kernels/seqmix_*.hip:
+#
+# * the residual stream is fp32 whatever the activation dtype; norms, router, softmax, the
+#   map combination and the per-head unit norm are fp32;
+# * per layer run the KV cache is ``k : [num_blocks, n_kv, block_size, maps * dim]`` and
+#   ``v : [num_blocks, n_kv, vdim, block_size]`` (V transposed per block-head, as above);
+# * a q / k head is laid out map after map: ``[map 0 (dim), map 1 (dim), ...]``.
+
+def rope_inv_freq(rot_dims: int, base: float, device=None) -> torch.Tensor:
+    """fp32 ``base^(-2i/rot_dims)``, i < rot_dims/2 (empty for rot_dims = 0)."""
+    i = torch.arange(rot_dims // 2, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / max(rot_dims, 1))).float().to(device)
+
+
+def rmsnorm32(x: torch.Tensor, w: torch.Tensor, eps: float, w_offset: float, out_dtype) -> torch.Tensor:
+    """fp32 ``x / sqrt(mean(x^2) + eps) * (w_offset + w)``, rounded once to ``out_dtype``."""
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * (w_offset + w.float())).to(out_dtype)
+
+
+def embed_scale_rmsnorm(tokens, table, scale: float, w, eps: float, w_offset: float, out_dtype):
+    """(norm(scale * E[tokens]) in ``out_dtype``, scale * E[tokens] in fp32)."""
+    residual = table.index_select(0, tokens.long()).float() * scale
+    return rmsnorm32(residual, w, eps, w_offset, out_dtype), residual
+
+
+def residual_add_rmsnorm32(residual, parts, w, eps: float, w_offset: float, out_dtype, gate=None, gated=None):
+    """``residual += sum(parts) [+ sigmoid(gate) * gated]`` in fp32, in place (the sublayer
+    outputs are summed first, then added); returns the norm of the new residual
+    (None when ``w`` is None).  ``gate`` : fp32 [T] logits, ``gated`` : [T, W]."""
+    total = None
+    for p in parts:
+        total = p.float() if total is None else total + p.float()
+    if gated is not None:
+        g = torch.sigmoid(gate.float())[:, None] * gated.float()
+        total = g if total is None else total + g
+    if total is not None:
+        residual.add_(total)
+    return None if w is None else rmsnorm32(residual, w, eps, w_offset, out_dtype)
+
+
+def rope_multi_kv_write(qkv, positions, slots, n_q: int, n_kv: int, maps: int, dim: int, vdim: int,
+                        inv_freq, k_cache, v_cache):
+    """Split a fused projection row ``[q | k | v | anything]``, rotate the first
+    ``2 * len(inv_freq)`` features of every map of every q / k head (feature i pairs with
+    i + rot/2; angle = position * inv_freq[i], fp32), scatter K / V into the paged cache of
+    this layer run.  Returns q ``[T, n_q, maps * dim]`` in the activation dtype."""
+    T = qkv.shape[0]
+    qw, kw = n_q * maps * dim, n_kv * maps * dim
+    q = qkv[:, :qw].float().reshape(T, n_q, maps, dim)
+    k = qkv[:, qw:qw + kw].float().reshape(T, n_kv, maps, dim)
+    v = qkv[:, qw + kw:qw + kw + n_kv * vdim].reshape(T, n_kv, vdim)
+    half = inv_freq.numel()
+    if half:
+        ang = positions.float()[:, None] * inv_freq.float()[None, :]
+        cos, sin = ang.cos()[:, None, None, :], ang.sin()[:, None, None, :]
+
+        def rot(x):
+            a, b, rest = x[..., :half], x[..., half:2 * half], x[..., 2 * half:]
+            return torch.cat([a * cos - b * sin, b * cos + a * sin, rest], dim=-1)
+        q, k = rot(q), rot(k)
+    bs = k_cache.shape[2]
+    blk, off = (slots // bs).long(), (slots % bs).long()
+    k_cache[blk, :, off] = k.reshape(T, n_kv, maps * dim).to(k_cache.dtype)
+    v_cache[blk, :, :, off] = v.to(v_cache.dtype)
+    return q.reshape(T, n_q, maps * dim).to(qkv.dtype)
+
+
+def multimap_attention(q, k_cache, v_cache, block_tables, q_start, seq_lens, scale: float, maps: int,
+                       lam: float, head_eps: float, out_scale: float, vdim: int):
+    """Causal GQA attention with ``maps`` softmax maps per head over shared values:
+    ``o = a_0 - lam * a_1`` (maps = 2; maps = 1: ``a_0``), then per head
+    ``o / sqrt(mean(o^2) + head_eps) * out_scale`` (``head_eps < 0``: only the scale).
+    Sequence b's query rows ``q_start[b]:q_start[b+1]`` are its last positions.  Returns
+    ``[T, n_q * vdim]``; fp32 math."""
+    T, n_q, qd = q.shape
+    dim = qd // maps
+    n_kv = k_cache.shape[1]
+    group = n_q // n_kv
+    bs = k_cache.shape[2]
+    out = torch.zeros(T, n_q, vdim, dtype=torch.float32, device=q.device)
+    for b in range(block_tables.shape[0]):
+        s, e = int(q_start[b]), int(q_start[b + 1])
+        if e <= s:
+            continue
+        ctx = int(seq_lens[b])
+        nblk = (ctx + bs - 1) // bs
+        ids = block_tables[b, :nblk].long()
+        k = k_cache[ids].permute(1, 0, 2, 3).reshape(n_kv, nblk * bs, qd)[:, :ctx].float()
+        v = v_cache[ids].permute(1, 0, 3, 2).reshape(n_kv, nblk * bs, vdim)[:, :ctx].float()
+        k, v = k.repeat_interleave(group, 0), v.repeat_interleave(group, 0)
+        qb = q[s:e].float().permute(1, 0, 2)
+        qpos = torch.arange(ctx - (e - s), ctx, device=q.device)[:, None]
+        hidden = torch.arange(ctx, device=q.device)[None, :] > qpos
+        o = None
+        for m in range(maps):
+            sc = torch.matmul(qb[..., m * dim:(m + 1) * dim], k[..., m * dim:(m + 1) * dim].transpose(1, 2)) * scale
+            a = torch.matmul(torch.softmax(sc.masked_fill(hidden, float("-inf")), -1), v)
+            o = a if m == 0 else o - lam * a
+        if head_eps >= 0:
+            o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + head_eps)
+        out[s:e] = (o * out_scale).permute(1, 0, 2)
+    return out.reshape(T, n_q * vdim).to(q.dtype)
+
+
+def act_fn(x: torch.Tensor, kind: str) -> torch.Tensor:
+    """"gelu_tanh": 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))); "relu2": max(z, 0)^2."""
+    z = x.float()
+    if kind == "gelu_tanh":
+        y = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
+    elif kind == "relu2":
+        y = torch.relu(z).pow(2)
+    else:
+        raise ValueError(f"unknown activation {kind!r}")
+    return y.to(x.dtype)
+
+
+def moe_route(h, router_w, router_b, top: int, gate_w=None):
+    """fp32 router: ``z = W h + b``; the ``top`` largest logits (ties: lowest index) and the
+    softmax over those only.  Returns (expert ids int32 [T, top], weights fp32 [T, top],
+    fp32 [T] logit of the always-on expert's gate ``gate_w . h`` or None)."""
+    hf = h.float()
+    z = hf @ router_w.float().t()
+    if router_b is not None:
+        z = z + router_b.float()
+    val, idx = torch.sort(z, dim=-1, descending=True, stable=True)
+    gate = None if gate_w is None else hf @ gate_w.float().reshape(-1)
+    return idx[:, :top].to(torch.int32), torch.softmax(val[:, :top], dim=-1), gate
+
+
+def moe_experts(h, up, down, idx, weights, kind: str = "relu2"):
+    """``sum_j weights[t, j] * down[e] act(up[e] h_t)``, e = idx[t, j]; up [E, ff, W],
+    down [E, W, ff].  Hidden activations are rounded to the activation dtype like a
+    projection's output; the weighted sum is returned in fp32 (it goes into the fp32 residual)."""
+    T, W = h.shape
+    out = torch.zeros(T, W, dtype=torch.float32, device=h.device)
+    for e in range(up.shape[0]):
+        rows, slot = (idx == e).nonzero(as_tuple=True)
+        if rows.numel() == 0:
+            continue
+        x = h.index_select(0, rows)
+        y = torch.nn.functional.linear(act_fn(torch.nn.functional.linear(x, up[e]), kind), down[e])
+        out.index_add_(0, rows, y.float() * weights[rows, slot][:, None])
+    return out

@@ -49,6 +49,7 @@ PYBIND11_MODULE(_bcg_runtime, m) {
       .def(py::init<int, int>(), py::arg("num_blocks"), py::arg("block_size"))
       .def("allocate", &BlockManager::allocate, py::arg("prompt"), py::arg("max_new_tokens"),
            py::arg("use_cache") = true)
+      .def("grow", &BlockManager::grow, py::arg("n"))
       .def("commit_prompt", &BlockManager::commit_prompt)
       .def("free", &BlockManager::free)
       .def("reset_cache", &BlockManager::reset_cache)

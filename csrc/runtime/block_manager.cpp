@@ -115,6 +115,19 @@ Allocation BlockManager::allocate(const std::vector<int32_t>& prompt, int max_ne
   return a;
 }
 
+std::vector<int> BlockManager::grow(int n) {
+  std::vector<int> out;
+  if (n <= 0 || n > num_free_blocks()) return out;
+  out.reserve(n);
+  for (int i = 0; i < n; ++i) {
+    int b = take_block();
+    meta_[b].ref = 1;
+    meta_[b].hashed = false;
+    out.push_back(b);
+  }
+  return out;
+}
+
 void BlockManager::commit_prompt(const std::vector<int>& blocks, const std::vector<int32_t>& prompt) {
   // register every full prompt block (content now resident in HBM)
   const int full = static_cast<int>(prompt.size()) / block_size_;

@@ -31,6 +31,9 @@ class BlockManager {
  public:
   BlockManager(int num_blocks, int block_size);
   Allocation allocate(const std::vector<int32_t>& prompt, int max_new_tokens, bool use_cache);
+  // `n` more blocks for a sequence whose length is not known at admission (token streams):
+  // all of them or none (empty result when fewer than `n` are free).
+  std::vector<int> grow(int n);
   void commit_prompt(const std::vector<int>& blocks, const std::vector<int32_t>& prompt);
   void free(const std::vector<int>& blocks);
   void reset_cache();
