@@ -92,6 +92,24 @@ def load_library(path: str = None) -> ctypes.CDLL:
                             c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "bcg_gemm_tile": [c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int)],
         "bcg_gemm_num_cfgs": [],
+        "bcg_embed_scale_rmsnorm": [c_void_p, c_void_p, c_float, c_void_p, c_float, c_float, c_void_p, c_void_p,
+                                    c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_residual_add_rmsnorm32": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+                                       c_float, c_void_p, c_int, c_int, c_int, c_void_p],
+        "bcg_act_fn": [c_void_p, c_void_p, c_int64, c_int, c_int64, c_int, c_int, c_void_p],
+        "bcg_rope_multi_kv_write": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                    c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_multimap_split_keys": [],
+        "bcg_multimap_attention": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                   c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                   c_float, c_float, c_float, c_float, c_int, c_void_p],
+        "bcg_moe_tile_rows": [],
+        "bcg_moe_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                          c_int, c_int, c_void_p],
+        "bcg_moe_align": [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
+        "bcg_moe_gemm": [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int,
+                         c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_moe_combine": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "bcg_guided_sample": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                               c_uint32, c_int, c_int, c_int, c_int, c_void_p],
@@ -553,7 +571,10 @@ def hip_ops() -> SimpleNamespace:
                                    out=residual)
         return residual.add_(linear_fp8(xq, xs, wq, ws))
 
-    return SimpleNamespace(name="hip", rmsnorm_fp8=rmsnorm_fp8, embed_rmsnorm_fp8=embed_rmsnorm_fp8,
+    from .seqmix import seqmix_ops
+    extra = seqmix_ops(lib, linear)
+
+    return SimpleNamespace(name="hip", **extra, rmsnorm_fp8=rmsnorm_fp8, embed_rmsnorm_fp8=embed_rmsnorm_fp8,
                            linear_fp8_residual=linear_fp8_residual, linear=linear, linear_silu=linear_silu, linear_residual=linear_residual,
                            gemm_nt=gemm_nt, gemm_plan=plan, prepare_device=prepare_device,
                            register_stream=register_stream, quant_fp8=quant_fp8, add_rmsnorm_fp8=add_rmsnorm_fp8,

@@ -161,6 +161,8 @@ def build_kernels(force: bool = False, verbose: bool = False) -> str:
     objdir = tempfile.mkdtemp(prefix="bcg_obj_", dir=os.path.dirname(target))
     flags = [f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC",
              "-fgpu-flush-denormals-to-zero", "-munsafe-fp-atomics",
+             # no packed fp32 VALU forms (the host pass warns that it does not know the feature)
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              f'-DBCG_SOURCE_HASH="{digest}"', f"-I{os.path.join(CSRC, 'kernels')}"]
     if os.environ.get("BCG_RESOURCE_USAGE"):
         flags.insert(0, "-Rpass-analysis=kernel-resource-usage")

@@ -1,0 +1,223 @@
+// Mixture-of-experts feed-forward with device-side routing (no host synchronisation):
+//
+//   route   : fp32 logits z = R h + b, the `top` largest (ties: lowest index), softmax over
+//             those only; also the fp32 logit of the always-on expert's gate
+//   align   : slots (token, j) bucketed by expert into tile-aligned position ranges
+//   gemm    : per position tile (one expert) C = A W_e^T on 16 x 16 MFMAs; "up" gathers token
+//             rows and applies the activation, "down" scatters rows back to their slots
+//   combine : out32[t] = sum_j weight[t, j] * y[slot(t, j)]   (fp32, fixed order)
+//
+// Position tiles are TM rows; a tile belongs to one expert (tile_expert, -1 = unused).
+#include <algorithm>
+
+#include "seqmix_common.h"
+
+namespace {
+
+constexpr int TM = 32, TN = 128, MAX_E = 256;
+
+template <typename T>
+__global__ __launch_bounds__(64) void route_kernel(const T* __restrict__ h, const float* __restrict__ rw,
+                                                   const float* __restrict__ rb, const float* __restrict__ gw,
+                                                   int* __restrict__ idx, float* __restrict__ wts,
+                                                   float* __restrict__ gate, int W, int E, int top) {
+  __shared__ float z[MAX_E];
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const T* row = h + static_cast<size_t>(t) * W;
+  for (int e = 0; e < E; ++e) {
+    float d = 0.f;
+    for (int i = lane; i < W; i += 64) d += Elem<T>::ld(row[i]) * rw[static_cast<size_t>(e) * W + i];
+    d = wave_sum(d);
+    if (lane == 0) z[e] = d + (rb ? rb[e] : 0.f);
+  }
+  if (gw != nullptr) {
+    float d = 0.f;
+    for (int i = lane; i < W; i += 64) d += Elem<T>::ld(row[i]) * gw[i];
+    d = wave_sum(d);
+    if (lane == 0) gate[t] = d;
+  }
+  __syncthreads();
+  if (lane == 0) {
+    float best0 = 0.f, den = 0.f;
+    for (int j = 0; j < top; ++j) {
+      int be = 0;
+      float bv = -INFINITY;
+      for (int e = 0; e < E; ++e)
+        if (z[e] > bv) { bv = z[e]; be = e; }
+      z[be] = -INFINITY;
+      if (j == 0) best0 = bv;
+      const float p = expf(bv - best0);
+      idx[t * top + j] = be;
+      wts[t * top + j] = p;
+      den += p;
+    }
+    for (int j = 0; j < top; ++j) wts[t * top + j] /= den;
+  }
+}
+
+__global__ __launch_bounds__(1024) void align_kernel(const int* __restrict__ idx, int n_slots, int E,
+                                                     int* __restrict__ sorted, int cap, int* __restrict__ tile_expert,
+                                                     int n_tiles) {
+  __shared__ int cnt[MAX_E], off[MAX_E + 1];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_slots; i += blockDim.x) {
+    const int e = idx[i];
+    if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
+  }
+  for (int i = threadIdx.x; i < cap; i += blockDim.x) sorted[i] = -1;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    off[0] = 0;
+    for (int e = 0; e < E; ++e) off[e + 1] = off[e] + (cnt[e] + TM - 1) / TM * TM;
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < n_tiles; t += blockDim.x) {
+    int who = -1;
+    for (int e = 0; e < E; ++e)
+      if (t * TM >= off[e] && t * TM < off[e + 1]) who = e;
+    tile_expert[t] = who;
+  }
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_slots; i += blockDim.x) {
+    const int e = idx[i];
+    if (e >= 0 && e < E) sorted[off[e] + atomicAdd(&cnt[e], 1)] = i;
+  }
+}
+
+// Position p of tile blockIdx.x: slot = sorted[p] (-1: padding).  gather: A row = a[(slot / top)]
+// (token rows), else a[p].  scatter: output row = slot, else p.  act 1: relu squared.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w,
+                                                       T* __restrict__ out, int64_t out_stride,
+                                                       const int* __restrict__ sorted,
+                                                       const int* __restrict__ tile_expert, int N, int K, int top,
+                                                       int gather, int scatter, int act, int vec) {
+  typedef typename Elem<T>::frag F;
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int p0 = blockIdx.x * TM, n0 = blockIdx.y * TN + 32 * wave;
+  if (n0 >= N) return;
+  const T* we = w + static_cast<size_t>(e) * N * K;
+  const T* arow[2];
+  int slot[2];
+  const T* wrow[2];
+  bool wok[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int p = p0 + 16 * i + col;
+    slot[i] = sorted[p];
+    const int64_t r = gather ? (slot[i] < 0 ? 0 : slot[i] / top) : p;
+    arow[i] = a + r * a_stride;
+    const int n = n0 + 16 * i + col;
+    wok[i] = n < N;
+    wrow[i] = we + static_cast<size_t>(wok[i] ? n : 0) * K;
+  }
+  f32x4 acc[2][2];  // [n tile][m tile]: lane holds C[m = col][n = 4 grp + i]
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k = 4 * grp; k < K; k += 16) {
+    F af[2], wf[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      af[i] = slot[i] >= 0 ? load_frag<T>(arow[i] + k, K - k, vec) : zero_frag<T>();
+      wf[i] = wok[i] ? load_frag<T>(wrow[i] + k, K - k, vec) : zero_frag<T>();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = mma16(wf[i], af[j], acc[i][j]);
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    if (slot[j] < 0) continue;
+    const int64_t r = scatter ? slot[j] : p0 + 16 * j + col;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + 16 * i + 4 * grp + q;
+        if (n < N) {
+          float v = acc[i][j][q];
+          if (act == 1) { v = fmaxf(v, 0.f); v *= v; }
+          out[r * out_stride + n] = Elem<T>::st(v);
+        }
+      }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ y, const float* __restrict__ wts,
+                                                      float* __restrict__ out, int W, int top) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float s = 0.f;
+    for (int j = 0; j < top; ++j) s += wts[t * top + j] * Elem<T>::ld(y[(static_cast<size_t>(t) * top + j) * W + c]);
+    out[static_cast<size_t>(t) * W + c] = s;
+  }
+}
+
+}  // namespace
+
+BCG_API int bcg_moe_tile_rows() { return TM; }
+
+BCG_API int bcg_moe_route(const void* h, const void* rw, const void* rb, const void* gw, void* idx, void* wts, void* gate,
+                          int T_, int W, int E, int top, int is_f32, void* stream) {
+  if (T_ <= 0) return 0;
+  if (E < 1 || E > MAX_E || top < 1 || top > E) return -2;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (is_f32)
+    route_kernel<float><<<T_, 64, 0, s>>>(static_cast<const float*>(h), static_cast<const float*>(rw), static_cast<const float*>(rb),
+                                         static_cast<const float*>(gw), static_cast<int*>(idx), static_cast<float*>(wts),
+                                         static_cast<float*>(gate), W, E, top);
+  else
+    route_kernel<bf16_t><<<T_, 64, 0, s>>>(static_cast<const bf16_t*>(h), static_cast<const float*>(rw), static_cast<const float*>(rb),
+                                          static_cast<const float*>(gw), static_cast<int*>(idx), static_cast<float*>(wts),
+                                          static_cast<float*>(gate), W, E, top);
+  return BCG_CHECK_LAUNCH();
+}
+
+// sorted: [cap] with cap = n_tiles * TM >= n_slots + E (TM - 1); tile_expert: [n_tiles].
+BCG_API int bcg_moe_align(const void* idx, int n_slots, int E, void* sorted, int cap, void* tile_expert, int n_tiles,
+                          void* stream) {
+  if (n_slots <= 0) return 0;
+  if (E < 1 || E > MAX_E || cap != n_tiles * TM || cap < n_slots + E * (TM - 1)) return -2;
+  align_kernel<<<1, 1024, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const int*>(idx), n_slots, E,
+                                                                 static_cast<int*>(sorted), cap,
+                                                                 static_cast<int*>(tile_expert), n_tiles);
+  return BCG_CHECK_LAUNCH();
+}
+
+BCG_API int bcg_moe_gemm(const void* a, int64_t a_stride, const void* w, void* out, int64_t out_stride, const void* sorted,
+                         const void* tile_expert, int n_tiles, int N, int K, int top, int gather, int scatter, int act,
+                         int is_f32, void* stream) {
+  if (n_tiles <= 0) return 0;
+  if (N < 1 || K < 1 || n_tiles > (1 << 24) || (N + TN - 1) / TN > 65535) return -2;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(n_tiles, (N + TN - 1) / TN);
+  const int vec = (K % 4 == 0 && a_stride % 4 == 0) ? 1 : 0;
+  if (is_f32)
+    moe_gemm_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(a), a_stride, static_cast<const float*>(w),
+                                               static_cast<float*>(out), out_stride, static_cast<const int*>(sorted),
+                                               static_cast<const int*>(tile_expert), N, K, top, gather, scatter, act, vec);
+  else
+    moe_gemm_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(a), a_stride, static_cast<const bf16_t*>(w),
+                                                static_cast<bf16_t*>(out), out_stride, static_cast<const int*>(sorted),
+                                                static_cast<const int*>(tile_expert), N, K, top, gather, scatter, act, vec);
+  return BCG_CHECK_LAUNCH();
+}
+
+BCG_API int bcg_moe_combine(const void* y, const void* wts, void* out, int T_, int W, int top, int is_f32, void* stream) {
+  if (T_ <= 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (is_f32)
+    combine_kernel<float><<<T_, 256, 0, s>>>(static_cast<const float*>(y), static_cast<const float*>(wts), static_cast<float*>(out), W, top);
+  else
+    combine_kernel<bf16_t><<<T_, 256, 0, s>>>(static_cast<const bf16_t*>(y), static_cast<const float*>(wts), static_cast<float*>(out), W, top);
+  return BCG_CHECK_LAUNCH();
+}
