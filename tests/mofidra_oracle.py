@@ -109,18 +109,22 @@ def layer_order(cfg):
     return list(range(loop["start"])) + span * loop["times"] + list(range(loop["stop"], n))
 
 
-def router_margin(cfg, sd, tokens):
-    """Smallest gap between a chosen and a not-chosen router logit over the sequence (a test
-    whose margin is tiny would compare two equally valid routings)."""
-    gaps = []
+def router_margins(cfg, sd, tokens):
+    """Per position, the smallest gap between a chosen and a not-chosen router logit over all
+    layer runs (a position whose margin is tiny has two equally valid routings)."""
+    gaps = [torch.full((len(tokens),), math.inf, dtype=F64)]
 
     def hook(h, prefix, f):
         if f is not None and f["kind"] == "moe" and f["router"]["top"] < f["router"]["experts"]:
             z = h @ sd[prefix + "router"].to(F64).T + sd[prefix + "router.b"].to(F64)
             s = torch.sort(z, -1, descending=True).values
-            gaps.append(float((s[:, f["router"]["top"] - 1] - s[:, f["router"]["top"]]).min()))
+            gaps.append(s[:, f["router"]["top"] - 1] - s[:, f["router"]["top"]])
     forward(cfg, sd, tokens, hook)
-    return min(gaps) if gaps else math.inf
+    return torch.stack(gaps).min(0).values
+
+
+def router_margin(cfg, sd, tokens):
+    return float(router_margins(cfg, sd, tokens).min())
 
 
 def forward(cfg, sd, tokens, hook=None, stream=None):

@@ -27,39 +27,54 @@ def case(request, tmp_path_factory):
     eng.shutdown()
 
 
+def _want(cfg, sd, toks):
+    """(oracle logits, positions whose routing is clear of a tie by more than bf16 rounding of the input)."""
+    return O.forward(cfg, sd, toks), O.router_margins(cfg, sd, toks) > 0.05
+
+
 def _close(got, want, dtype):
+    want, clear = want
     got = got.double().cpu()
     if dtype == "float32":
         torch.testing.assert_close(got, want, atol=3e-3, rtol=3e-3)
-    else:  # bf16 activations: error relative to the spread of the logits
+    else:  # bf16 activations: error relative to the spread of the logits, where the routing cannot flip
         err = (got - want).pow(2).mean(-1).sqrt() / want.std()
-        assert float(err.max()) < 0.08, float(err.max())
+        assert float(err[clear].max() if clear.any() else 0.0) < 0.08, float(err[clear].max())
+        assert float(err.median()) < 0.02
+
+
+def _rows(want, sl):
+    return want[0][sl], want[1][sl]
+
+
+def _cat(parts):
+    return torch.cat([p[0] for p in parts]), torch.cat([p[1] for p in parts])
 
 
 def test_whole_prompt_every_position(case):
     cfg, sd, eng, dtype = case
     toks = C.tokens(150, cfg["vocab"], 1)
     got = eng.stream_step([("a", toks, list(range(150)))], end=["a"])
-    _close(got, O.forward(cfg, sd, toks), dtype)
+    _close(got, _want(cfg, sd, toks), dtype)
 
 
 def test_portions_then_single_tokens(case):
     cfg, sd, eng, dtype = case
     toks = C.tokens(140, cfg["vocab"], 2)
-    want = O.forward(cfg, sd, toks)
+    want = _want(cfg, sd, toks)
     at = 0
     for s in [2, 3, 64, 1, 17, 2, 1]:
-        _close(eng.stream_step([("p", toks[at:at + s], list(range(s)))]), want[at:at + s], dtype)
+        _close(eng.stream_step([("p", toks[at:at + s], list(range(s)))]), _rows(want, slice(at, at + s)), dtype)
         at += s
-    for p in range(at, 140):
-        _close(eng.stream_step([("p", toks[p:p + 1], [0])], end=["p"] if p == 139 else []), want[p:p + 1], dtype)
+    got = [eng.stream_step([("p", toks[p:p + 1], [0])], end=["p"] if p == 139 else []) for p in range(at, 140)]
+    _close(torch.cat(got), _rows(want, slice(at, 140)), dtype)
 
 
 def test_mixed_batches_and_reuse(case):
     cfg, sd, eng, dtype = case
     lens = [70, 33, 18, 64, 41, 90, 5, 36, 120]
     reqs = {f"r{i}": C.tokens(n, cfg["vocab"], 10 + i) for i, n in enumerate(lens)}
-    want = {k: O.forward(cfg, sd, t) for k, t in reqs.items()}
+    want = {k: _want(cfg, sd, t) for k, t in reqs.items()}
     at = {k: 0 for k in reqs}
     waiting, live, step = list(reqs), [], 0
     free_at_start = eng.blocks.num_free_blocks
@@ -71,11 +86,11 @@ def test_mixed_batches_and_reuse(case):
             take = [1, 2, 16, 7, 1, 19][(step + j) % 6] if at[k] > 0 else [20, 3, 16][j % 3]
             take = min(take, len(reqs[k]) - at[k])
             entries.append((k, reqs[k][at[k]:at[k] + take], list(range(take))))
-            expect.append(want[k][at[k]:at[k] + take])
+            expect.append(_rows(want[k], slice(at[k], at[k] + take)))
             at[k] += take
             if at[k] == len(reqs[k]):
                 end.append(k)
-        _close(eng.stream_step(entries, end), torch.cat(expect), dtype)
+        _close(eng.stream_step(entries, end), _cat(expect), dtype)
         live = [k for k in live if k not in end]
         step += 1
     assert eng.blocks.num_free_blocks == free_at_start and not any(eng.slots)
