@@ -1,0 +1,212 @@
+"""Prefill / decode throughput of the Mofidra family beside the Qwen3-style decoder at equal
+layer sizes (random weights, synthetic tokens), and the hot kernels of both against their
+rooflines.  ``bench.py --family-compare`` prints the result as one JSON line.
+
+Equal size: same width, layers, query / KV heads, 128 features per query head (Mofidra: two
+64-wide maps), 128 value features, the same feed-forward width (the decoder's SwiGLU has three
+matrices, the dense gelu layer two; the MoE variant routes top-2 of 8 experts of ff/4 plus an
+always-on expert of ff/2, i.e. the dense layer's active parameters).
+
+Rooflines: 2.5 PFLOP/s dense bf16 MFMA, 8 TB/s HBM.  A kernel's ``roof_frac`` is
+max(flops / peak, bytes / bandwidth) / measured time.
+"""
+
+import json
+import time
+
+import torch
+
+from ..models.config import MofidraConfig, ModelConfig
+from ..models.mofidra import MofidraModel
+from ..models.transformer import AttnMeta, DecoderModel
+from ..ops import get_ops
+
+PEAK_FLOPS, PEAK_BW = 2.5e15, 8.0e12
+BS = 16
+
+SIZES = {
+    "w2048": dict(width=2048, layers=4, heads=16, kv_heads=4, ff=8192, vocab=32768),
+    "w4096": dict(width=4096, layers=4, heads=32, kv_heads=8, ff=12288, vocab=32768),
+}
+
+
+def mofidra_config(s, moe: bool) -> MofidraConfig:
+    mixer = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": 64, "vdim": 128, "scale": 0.125, "diff": 0.5,
+             "rot": {"dims": 64, "base": 1e6}}
+    mlp = ({"kind": "moe", "expert": {"ff": s["ff"] // 4}, "router": {"experts": 8, "top": 2}, "shared": {"ff": s["ff"] // 2}}
+           if moe else {"kind": "dense", "ff": s["ff"]})
+    return MofidraConfig.from_dict({"architecture": "Mofidra", "width": s["width"], "vocab": s["vocab"],
+                                    "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
+                                    "layers": [{"type": "attention", "mixer": mixer, "mlp": mlp}] * s["layers"]},
+                                   "mofidra-bench")
+
+
+def decoder_config(s) -> ModelConfig:
+    return ModelConfig("decoder-bench", "qwen3", s["width"], s["layers"], s["heads"], s["kv_heads"], 128, s["ff"],
+                       s["vocab"], qk_norm=True)
+
+
+def step_meta(n_seq, ctx, q_len, tile_rows, device, split_single):
+    """Packed step: `n_seq` sequences of `ctx` resident tokens, the last `q_len` are this step's."""
+    nblk = (ctx + BS - 1) // BS
+    tables = (torch.arange(n_seq * nblk, dtype=torch.int32).view(n_seq, nblk) + 1)
+    pos = torch.arange(ctx - q_len, ctx).repeat(n_seq)
+    seq = torch.arange(n_seq).repeat_interleave(q_len)
+    slots = tables[seq, pos // BS].long() * BS + pos % BS
+    q_start = torch.arange(n_seq + 1) * q_len
+    i32 = torch.int32
+    decode = q_len == 1
+    tiles, single = [], []
+    if not decode:
+        for b in range(n_seq):
+            for t in range(b * q_len, (b + 1) * q_len, tile_rows):
+                tiles.append((ctx - ((b + 1) * q_len - t), b, t, min(t + tile_rows, (b + 1) * q_len)))
+        tiles.sort(key=lambda x: -x[0])
+    meta = AttnMeta(positions=pos.to(i32).to(device), slots=slots.to(i32).to(device), block_tables=tables.to(device),
+                    seq_lens=torch.full((n_seq,), ctx, dtype=i32, device=device), q_start=q_start.to(i32).to(device),
+                    max_q_len=q_len, decode=decode, tile_rows=tile_rows,
+                    logits_idx=(q_start[1:] - 1).long().to(device),
+                    tiles=torch.tensor([t[1:] for t in tiles], dtype=i32, device=device).reshape(-1, 3),
+                    single=torch.zeros(0, 2, dtype=i32, device=device) if split_single else None)
+    return meta, n_seq * nblk + 1
+
+
+def _time(fn, warmup=3, iters=10):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / iters
+
+
+def _graph_time(fn, iters=30):
+    fn()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    return _time(g.replay, warmup=3, iters=iters)
+
+
+def model_throughput(model, prefill=(8, 1024), decode=(64, 1024)):
+    dev = model.device
+    tile_rows = getattr(model, "prefill_tile_rows", None) or model.ops.prefill_tile_rows(model.hd, False, 1024)
+    split = getattr(model, "split_single_rows", False)
+    out = {}
+    n, s = prefill
+    meta, nb = step_meta(n, s, s, tile_rows, dev, split)
+    k, v = model.alloc_kv(max(nb, decode[0] * ((decode[1] + BS - 1) // BS) + 1), BS, torch.bfloat16)
+    tokens = torch.randint(0, model.cfg.vocab_size, (n * s,), dtype=torch.int32, device=dev)
+    t = _time(lambda: model.forward(tokens, meta, k, v), iters=5)
+    out["prefill_tokens_per_s"] = round(n * s / t)
+    out["prefill_ms"] = round(t * 1e3, 3)
+    b, ctx = decode
+    dmeta, _ = step_meta(b, ctx, 1, tile_rows, dev, split)
+    dmeta.logits_idx = None
+    dtok = torch.randint(0, model.cfg.vocab_size, (b,), dtype=torch.int32, device=dev)
+    t = _graph_time(lambda: model.forward(dtok, dmeta, k, v))
+    out["decode_tokens_per_s"] = round(b / t)
+    out["decode_ms"] = round(t * 1e3, 3)
+    return out
+
+
+def _roof(flops, bytes_, t):
+    return round(max(flops / PEAK_FLOPS, bytes_ / PEAK_BW) / t, 4)
+
+
+def kernel_pairs(s, dev):
+    """Like kernels of the two families at the same shapes: time and fraction of the roofline."""
+    ops = get_ops("hip")
+    H, G, W = s["heads"], s["kv_heads"], s["width"]
+    bf = torch.bfloat16
+    out = {}
+    # ---- prefill attention: 8 x 1024 tokens ----
+    n, ctx = 8, 1024
+    T = n * ctx
+    flops = 2 * H * (128 + 128) * n * ctx * ctx / 2   # decoder: QK^T over 128 features + PV over 128 values, causal half
+    kv_bytes = n * ctx * G * 256 * 2
+    io = T * H * 256 * 2 + kv_bytes
+    meta, nb = step_meta(n, ctx, ctx, 64, dev, True)
+    q = torch.randn(T, H, 128, device=dev, dtype=bf)
+    kc, vc = torch.randn(nb, G, BS, 128, device=dev, dtype=bf), torch.randn(nb, G, 128, BS, device=dev, dtype=bf)
+    t = _time(lambda: ops.multimap_attention(q, kc, vc, meta, 0.125, 2, 0.4, 1e-5, 0.5, 128))
+    out["prefill_attention"] = {"mofidra_ms": round(t * 1e3, 3), "mofidra_roof_frac": _roof(1.5 * flops, io, t)}  # two maps: PV twice
+    rows = ops.prefill_tile_rows(128, False, ctx // BS)
+    meta_d, _ = step_meta(n, ctx, ctx, rows, dev, False)
+    kd, vd = kc.unsqueeze(0).contiguous(), vc.unsqueeze(0).contiguous()
+    t = _time(lambda: ops.paged_attention_prefill(q, kd, vd, 0, meta_d.block_tables, meta_d.q_start, meta_d.seq_lens,
+                                                  0.088, ctx, meta_d.tiles, tile_rows=rows))
+    out["prefill_attention"].update({"decoder_ms": round(t * 1e3, 3), "decoder_roof_frac": _roof(flops, io, t)})
+    # ---- decode attention: 64 rows x 1024 context ----
+    b = 64
+    dmeta, nb = step_meta(b, ctx, 1, 64, dev, True)
+    kc, vc = torch.randn(nb, G, BS, 128, device=dev, dtype=bf), torch.randn(nb, G, 128, BS, device=dev, dtype=bf)
+    qd = torch.randn(b, H, 128, device=dev, dtype=bf)
+    kv_bytes = b * ctx * G * 256 * 2
+    dflops = 2 * H * 256 * b * ctx
+    t = _graph_time(lambda: ops.multimap_attention(qd, kc, vc, dmeta, 0.125, 2, 0.4, 1e-5, 0.5, 128), iters=50)
+    out["decode_attention"] = {"mofidra_ms": round(t * 1e3, 4), "mofidra_roof_frac": _roof(dflops * 1.5, kv_bytes, t)}
+    kd, vd = kc.unsqueeze(0).contiguous(), vc.unsqueeze(0).contiguous()
+    t = _graph_time(lambda: ops.paged_attention_decode(qd, kd, vd, 0, dmeta.block_tables, dmeta.seq_lens, 0.088), iters=50)
+    out["decode_attention"].update({"decoder_ms": round(t * 1e3, 4), "decoder_roof_frac": _roof(dflops, kv_bytes, t)})
+    # ---- routed experts (grouped GEMM) beside the dense projection of the same active FLOPs ----
+    E, top, ff = 8, 2, s["ff"] // 4
+    for name, T in (("prefill", 8192), ("decode", 64)):
+        h = torch.randn(T, W, device=dev, dtype=bf)
+        up = torch.randn(E, ff, W, device=dev, dtype=bf) * 0.02
+        down = torch.randn(E, W, ff, device=dev, dtype=bf) * 0.02
+        rw, rb = torch.randn(E, W, device=dev) * 0.02, torch.zeros(E, device=dev)
+        idx, wts, _ = ops.moe_route(h, rw, rb, top)
+        flops = 2 * 2 * T * top * ff * W
+        wbytes = 2 * E * ff * W * 2 + T * W * 2 * (2 + 2 * top)
+        t = _time(lambda: ops.moe_experts(h, up, down, idx, wts, "relu2"), iters=20)
+        wd_up = torch.randn(top * ff, W, device=dev, dtype=bf) * 0.02
+        wd_down = torch.randn(W, top * ff, device=dev, dtype=bf) * 0.02
+        t2 = _time(lambda: ops.linear(ops.linear(h, wd_up), wd_down), iters=20)
+        out[f"experts_{name}"] = {"mofidra_ms": round(t * 1e3, 4), "mofidra_roof_frac": _roof(flops, wbytes, t),
+                                  "dense_gemm_ms": round(t2 * 1e3, 4),
+                                  "dense_gemm_roof_frac": _roof(flops, 2 * top * ff * W * 2 + T * W * 4, t2)}
+    # ---- residual add + norm: fp32 stream against the bf16 stream ----
+    T = 8192
+    x32, p = torch.randn(T, W, device=dev), torch.randn(T, W, device=dev, dtype=bf)
+    w32 = torch.zeros(W, device=dev)
+    t = _time(lambda: ops.residual_add_rmsnorm32(x32, [p, p], w32, 1e-5, 1.0, bf), iters=20)
+    out["residual_norm"] = {"mofidra_ms": round(t * 1e3, 4), "mofidra_roof_frac": _roof(0, T * W * (4 + 4 + 2 + 2 + 2), t)}
+    xb, wb = torch.randn(T, W, device=dev, dtype=bf), torch.ones(W, device=dev, dtype=bf)
+    t = _time(lambda: ops.add_rmsnorm(p, xb, wb, 1e-5), iters=20)
+    out["residual_norm"].update({"decoder_ms": round(t * 1e3, 4), "decoder_roof_frac": _roof(0, T * W * (2 + 2 + 2 + 2), t)})
+    return out
+
+
+def run(sizes=("w2048", "w4096"), kernels=True) -> dict:
+    dev = torch.device("cuda", torch.cuda.current_device())
+    ops = get_ops("hip")
+    ops.prepare_device(dev)
+    result = {"metric": "family_compare", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "sizes": {}}
+    with torch.no_grad():
+        for name in sizes:
+            s = SIZES[name]
+            entry = {}
+            for label, build in (("mofidra_dense", lambda: MofidraModel(mofidra_config(s, False), ops, dev)),
+                                 ("mofidra_moe", lambda: MofidraModel(mofidra_config(s, True), ops, dev)),
+                                 ("decoder", lambda: DecoderModel(decoder_config(s), ops, dev))):
+                model = build()
+                model.init_random(seed=1, std=0.02)
+                entry[label] = model_throughput(model)
+                del model
+                torch.cuda.empty_cache()
+            if kernels:
+                entry["kernels"] = kernel_pairs(s, dev)
+            result["sizes"][name] = entry
+    return result
+
+
+if __name__ == "__main__":
+    print(json.dumps(run()))
