@@ -38,7 +38,6 @@ class MofidraModel:
     split_single_rows = True
     logits_dtype = torch.float32
     supports_cascade = False
-    prefill_tile_rows = 64      # query rows per prefill attention tile (4 waves x 16 rows)
 
     def __init__(self, cfg: MofidraConfig, ops, device, dtype=torch.bfloat16, tp: Optional[TPGroup] = None,
                  quant: Optional[str] = None):
@@ -56,6 +55,9 @@ class MofidraModel:
         self.hd = max(max(l.mixer.maps * l.mixer.dim, l.mixer.vdim) for l in cfg.layers)
         self.inter = max([l.mlp.ff * max(1, l.mlp.top) + l.mlp.shared_ff for l in cfg.layers if l.mlp] or [0])
         self.vocab_local = cfg.vocab_size
+        # query rows per prefill attention tile: what the backend's kernel takes for the largest heads
+        rows_fn = getattr(ops, "multimap_tile_rows", None)
+        self.prefill_tile_rows = min([rows_fn(l.mixer.dim, l.mixer.vdim) for l in cfg.layers]) if rows_fn else 64
 
     # ------------------------------------------------------------- KV cache
     def kv_block_bytes(self, block_size: int, dtype) -> int:

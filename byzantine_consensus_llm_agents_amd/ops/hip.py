@@ -102,7 +102,7 @@ def load_library(path: str = None) -> ctypes.CDLL:
         "bcg_multimap_split_keys": [],
         "bcg_multimap_attention": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                    c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                   c_float, c_float, c_float, c_float, c_int, c_void_p],
+                                   c_float, c_float, c_float, c_float, c_int, c_int, c_void_p],
         "bcg_moe_tile_rows": [],
         "bcg_moe_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                           c_int, c_int, c_void_p],

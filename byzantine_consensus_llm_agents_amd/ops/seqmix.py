@@ -96,6 +96,28 @@ def seqmix_ops(lib, linear):
              "KV cache: K [NB, G, BS, maps dim], V [NB, G, vdim, BS], BS % 16 == 0")
         return NB, BS
 
+    def kv_from_logical(k, v):
+        """The cache tensors the kernels read, from logical K [NB, G, BS, KD] / V [NB, G, vdim, BS]
+        (tests, tools): with KD % 4 == 0 every (page, head) slab is stored fragment-major, K as
+        [KD / 4][BS][4] and V as [BS / 4][vdim][4]; the shapes stay the logical ones."""
+        NB, G, BS, KD = k.shape
+        if KD % 4:
+            return k.contiguous(), v.contiguous()
+        vd = v.shape[2]
+        kp = k.reshape(NB, G, BS, KD // 4, 4).permute(0, 1, 3, 2, 4).contiguous().view(NB, G, BS, KD)
+        vp = v.reshape(NB, G, vd, BS // 4, 4).permute(0, 1, 3, 2, 4).contiguous().view(NB, G, vd, BS)
+        return kp, vp
+
+    def kv_to_logical(k, v):
+        """Inverse of `kv_from_logical`."""
+        NB, G, BS, KD = k.shape
+        if KD % 4:
+            return k, v
+        vd = v.shape[2]
+        kl = k.reshape(NB, G, KD // 4, BS, 4).permute(0, 1, 3, 2, 4).contiguous().view(NB, G, BS, KD)
+        vl = v.reshape(NB, G, BS // 4, vd, 4).permute(0, 1, 3, 2, 4).contiguous().view(NB, G, vd, BS)
+        return kl, vl
+
     def rope_multi_kv_write(qkv, positions, slots, n_q, n_kv, maps, dim, vdim, inv_freq, k_cache, v_cache):
         T = qkv.shape[0]
         qw, kw, vw = n_q * maps * dim, n_kv * maps * dim, n_kv * vdim
@@ -110,6 +132,10 @@ def seqmix_ops(lib, linear):
                                            _p(k_cache), _p(v_cache), T, n_q, n_kv, maps, dim, vdim, BS, NB, _act(qkv),
                                            _stream()), "rope_multi_kv_write")
         return q
+
+    def multimap_tile_rows(dim, vdim):
+        """Query rows per prefill tile (the tile table the engine builds) for these head sizes."""
+        return 64  # four waves x 16 rows
 
     def multimap_attention(q, k_cache, v_cache, meta, scale, maps, lam, head_eps, out_scale, vdim):
         """Prefill tiles (``meta.tiles``) on the MFMA kernel, one-token rows (``meta.single``, or
@@ -126,7 +152,9 @@ def seqmix_ops(lib, linear):
              and lens.is_contiguous() and lens.numel() == bt.shape[0], "block tables int32 [B, max_blocks], lens int32 [B]")
         out = torch.empty(T, H * vdim, dtype=q.dtype, device=q.device)
         f32 = _act(q)
-        common = (H, G, maps, dim, vdim, BS, NB, scale, lam, head_eps, out_scale, f32, _stream())
+        tile_rows = meta.tile_rows if not meta.decode else 64
+        _req(tile_rows == 64, "prefill tiles: 64 query rows")
+        common = (H, G, maps, dim, vdim, BS, NB, scale, lam, head_eps, out_scale, tile_rows, f32, _stream())
 
         def decode(work, n_items):
             n_splits = max(1, (bt.shape[1] * BS + split_keys - 1) // split_keys)
@@ -195,4 +223,5 @@ def seqmix_ops(lib, linear):
 
     return dict(embed_scale_rmsnorm=embed_scale_rmsnorm, residual_add_rmsnorm32=residual_add_rmsnorm32,
                 rmsnorm32=rmsnorm32, act_fn=act_fn, rope_multi_kv_write=rope_multi_kv_write,
-                multimap_attention=multimap_attention, moe_route=moe_route, moe_experts=moe_experts)
+                kv_from_logical=kv_from_logical, kv_to_logical=kv_to_logical,
+                multimap_attention=multimap_attention, multimap_tile_rows=multimap_tile_rows, moe_route=moe_route, moe_experts=moe_experts)

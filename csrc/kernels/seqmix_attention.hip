@@ -3,8 +3,12 @@
 //   head h, map m:  a_m = softmax(scale q_m K_m^T) V      (every map over the SAME values)
 //   o = a_0 - lam a_1   (maps = 2;  maps = 1: a_0),   o <- o / sqrt(mean(o^2) + eps) * out_scale
 //
-// Cache of one layer run: K [NB, G, BS, maps dim], V [NB, G, vdim, BS] (V transposed per
-// block-head: 16 consecutive keys of one value feature are contiguous).  BS is a multiple of 16.
+// Cache of one layer run: K [NB, G, BS, maps dim], V [NB, G, vdim, BS] logically.  With `swz`
+// (maps dim a multiple of 4) a (page, KV head) slab is stored fragment-major, so that the 64
+// lanes of one MFMA operand load read 512 contiguous bytes instead of 64 scattered 8-byte pieces:
+//   K slab [maps dim / 4][BS][4]  (4 features of one key, key after key, feature group after group)
+//   V slab [BS / 4][vdim][4]      (4 keys of one value feature, feature after feature, key group after group)
+// BS is a multiple of 16.
 //
 // prefill_kernel: a work tile is <= 64 query rows of one sequence (4 waves x 16 rows) for one
 // query head.  Per 16 keys a wave computes S^T = K Q^T (keys x queries) with 16 x 16 MFMAs, so
@@ -13,10 +17,12 @@
 // (reduced over the 4 lane groups).  K / V^T fragments are read straight from the cache
 // (a lane's share of an operand is 4 consecutive elements of one cache row).
 //
-// decode_kernel: one wave per (item, head, 256-key split); a lane scores one key per 64-key
-// chunk (q in LDS, fp32), the probabilities go through LDS and every lane then owns value
-// features e, e + 64, ... reading 16 contiguous keys of its V^T row per page.  The split
-// size is fixed, so a row's result does not depend on what else is in the batch.
+// The bf16 instance for heads up to 64 / 128 wide takes 32 keys per iteration and prefetches
+// the next iteration's K fragments in registers.
+//
+// decode_mfma_kernel: single-token rows.  The 16 MFMA columns hold the query heads that share
+// one KV head (GQA packing), so the cache is read once per KV head; one wave per 128-key split.
+// The split size is fixed, so a row's result does not depend on what else is in the batch.
 // decode_merge_kernel merges the splits and applies the map combination + head norm.
 #include <algorithm>
 
@@ -24,7 +30,7 @@
 
 namespace {
 
-constexpr int SPLIT_KEYS = 256;
+constexpr int SPLIT_KEYS = 128;
 
 struct AttnArgs {
   const void* q;            // [T, H, maps dim]
@@ -39,12 +45,175 @@ struct AttnArgs {
   int max_blocks, H, G, maps, dim, vdim, BS, num_blocks, n_splits;
   float scale, lam, head_eps, out_scale;
   int vec_k, vec_v;         // rows of K / V^T are aligned for 4-element vector loads
+  int swz;                  // fragment-major slabs (see the top of the file)
 };
 
-template <typename T, int KC, int VT>
+// The key loop shared by both kernels: keys [k_begin, k_last] of one sequence for the 16 query
+// columns of a wave (column = a query row of one head, or a query head of one token).
+//   limit      per lane: the last key its column may see;  limit_min: the smallest over the wave
+//   KT         16-key tiles per iteration (one softmax update and one rescale per iteration)
+//   PF         the next iteration's K fragments are loaded before this iteration's products and
+//              this iteration's V^T fragments before its QK^T products (loads fly under the MFMAs)
+//   FULL       whole, aligned fragments only (no branch around any load)
+// Everything that does not depend on the lane stays scalar: the page lookup and the slab base go
+// to SGPRs, a lane adds a 32-bit offset that is fixed for the whole loop.  Scores are kept in the
+// log2 domain (scale * log2 e folded into one multiply, v_exp_f32 directly).
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL>
+__device__ __forceinline__ void attend_range(const AttnArgs& a, int g, const typename Elem<T>::frag (&qf)[2][KC],
+                                             int limit, int limit_min, int k_begin, int k_last,
+                                             const int* __restrict__ table, f32x4 (&acc)[2][VT], float (&mx)[2],
+                                             float (&den)[2]) {
+  typedef typename Elem<T>::frag F;
+  const int lane = threadIdx.x & 63, col = lane & 15, grp = lane >> 4;
+  const int KD = a.maps * a.dim;
+  const int kc = (a.dim + 15) >> 4, vt = (a.vdim + 15) >> 4;
+  const bool vec_k = a.vec_k && (a.dim & 3) == 0;
+  const float sc = a.scale * 1.4426950408889634f;
+  // lane offsets inside a (page, KV head) slab; the slab base and the key offset are wave-uniform
+  uint32_t koffs[2][KC], voffs[VT];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int f = 16 * c + 4 * grp;        // this lane: key col, features m dim + f .. + 3
+      koffs[m][c] = a.swz ? (((m * a.dim + f) >> 2) * a.BS + col) * 4 : col * KD + m * a.dim + f;
+    }
+#pragma unroll
+  for (int t = 0; t < VT; ++t) {
+    const int e = 16 * t + col;              // this lane: value feature e, keys 4 grp .. + 3
+    voffs[t] = a.swz ? (grp * a.vdim + e) * 4 : e * a.BS + 4 * grp;
+  }
+  const int k_mul = a.swz ? 4 : KD, v_mul = a.swz ? a.vdim : 1;   // slab offset per key of the tile's first key
+  const T* kc_base = static_cast<const T*>(a.k_cache);
+  const T* vc_base = static_cast<const T*>(a.v_cache);
+  const size_t k_slab = static_cast<size_t>(a.BS) * KD, v_slab = static_cast<size_t>(a.BS) * a.vdim;
+
+  // tiles past the sequence read some valid page: every one of their keys is masked
+  auto slabs = [&](int key0, const T*& kp, const T*& vp) {
+    const int idx = min(key0 / a.BS, a.max_blocks - 1);
+    int page = table[idx];
+    page = (page < 0 || page >= a.num_blocks) ? 0 : page;
+    const size_t base = static_cast<size_t>(page) * a.G + g;
+    const int koff = key0 - (key0 / a.BS) * a.BS;
+    kp = kc_base + base * k_slab + koff * k_mul;
+    vp = vc_base + base * v_slab + koff * v_mul;
+  };
+  auto load_k = [&](int key0, F (&kf)[KT][2][KC]) {
+#pragma unroll
+    for (int u = 0; u < KT; ++u) {
+      const T *kp, *vp;
+      slabs(key0 + 16 * u, kp, vp);
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int c = 0; c < KC; ++c)
+          kf[u][m][c] = (m < a.maps && c < kc) ? load_frag_t<T, FULL>(kp + koffs[m][c], a.dim - (16 * c + 4 * grp), vec_k)
+                                               : zero_frag<T>();
+    }
+  };
+
+  F kn[KT][2][KC];
+  if (PF) load_k(k_begin, kn);
+  for (int key0 = k_begin; key0 <= k_last; key0 += 16 * KT) {
+    F vf[PF ? KT : 1][PF ? VT : 1];
+    auto load_v = [&](int u, int t) {
+      const T *kp, *vp;
+      slabs(key0 + 16 * u, kp, vp);
+      return (t < vt && 16 * t + col < a.vdim) ? load_frag_t<T, FULL>(vp + voffs[t], 4, a.vec_v) : zero_frag<T>();
+    };
+    if constexpr (PF) {
+#pragma unroll
+      for (int u = 0; u < KT; ++u)
+#pragma unroll
+        for (int t = 0; t < VT; ++t) vf[u][t] = load_v(u, t);
+    }
+    F kf[KT][2][KC];
+    if (PF) {
+#pragma unroll
+      for (int u = 0; u < KT; ++u)
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+          for (int c = 0; c < KC; ++c) kf[u][m][c] = kn[u][m][c];
+      if (key0 + 16 * KT <= k_last) load_k(key0 + 16 * KT, kn);
+    } else {
+      load_k(key0, kf);
+    }
+    // ---- S^T = K Q^T ----
+    f32x4 s[KT][2];
+#pragma unroll
+    for (int u = 0; u < KT; ++u)
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+        s[u][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (m < a.maps) {
+#pragma unroll
+          for (int c = 0; c < KC; ++c)
+            if (c < kc) s[u][m] = mma16(kf[u][m][c], qf[m][c], s[u][m]);
+        }
+      }
+    // ---- online softmax per query column; lane holds keys key0 + 16 u + 4 grp + i ----
+    const bool masked = key0 + 16 * KT - 1 > limit_min;     // (wave-uniform) some key of the iteration is hidden
+    F pf[KT][2];
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      if (m >= a.maps) {
+#pragma unroll
+        for (int u = 0; u < KT; ++u) pf[u][m] = zero_frag<T>();
+        continue;
+      }
+      float v[KT][4], bm = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < KT; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[u][i] = s[u][m][i] * sc;
+          if (masked && key0 + 16 * u + 4 * grp + i > limit) v[u][i] = -INFINITY;
+          bm = fmaxf(bm, v[u][i]);
+        }
+      bm = fmaxf(bm, __shfl_xor(bm, 16, WAVE));
+      bm = fmaxf(bm, __shfl_xor(bm, 32, WAVE));
+      const float m_new = fmaxf(mx[m], bm);                 // finite: the range's first key is visible
+      float ps = 0.f;
+#pragma unroll
+      for (int u = 0; u < KT; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[u][i] = __builtin_amdgcn_exp2f(v[u][i] - m_new);
+          ps += v[u][i];
+        }
+      ps += __shfl_xor(ps, 16, WAVE);
+      ps += __shfl_xor(ps, 32, WAVE);
+      if (__any(m_new > mx[m])) {                           // (wave-uniform) the running maximum moved
+        const float alpha = __builtin_amdgcn_exp2f(mx[m] - m_new);
+        den[m] *= alpha;
+#pragma unroll
+        for (int t = 0; t < VT; ++t)
+          if (t < vt) acc[m][t] *= alpha;
+      }
+      den[m] += ps;
+      mx[m] = m_new;
+#pragma unroll
+      for (int u = 0; u < KT; ++u) pf[u][m] = Elem<T>::pack(v[u][0], v[u][1], v[u][2], v[u][3]);
+    }
+    // ---- O^T += V^T P^T ----
+#pragma unroll
+    for (int u = 0; u < KT; ++u)
+#pragma unroll
+      for (int t = 0; t < VT; ++t)
+        if (t < vt) {
+          F x;
+          if constexpr (PF) x = vf[u][t]; else x = load_v(u, t);
+          acc[0][t] = mma16(x, pf[u][0], acc[0][t]);
+          if (a.maps > 1) acc[1][t] = mma16(x, pf[u][1], acc[1][t]);
+        }
+  }
+}
+
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL>
 __global__ __launch_bounds__(256) void prefill_kernel(AttnArgs a) {
   typedef typename Elem<T>::frag F;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col = lane & 15, grp = lane >> 4;
   const int h = blockIdx.y, g = h / (a.H / a.G);
   const int seq = a.work[3 * blockIdx.x], row0 = a.work[3 * blockIdx.x + 1] + 16 * wave, row_end = a.work[3 * blockIdx.x + 2];
@@ -53,11 +222,11 @@ __global__ __launch_bounds__(256) void prefill_kernel(AttnArgs a) {
   const int n_rows = min(16, row_end - row0);
   const int row = row0 + min(col, n_rows - 1);             // columns past the tile repeat its last row (never stored)
   const int pos = ctx - (q_end - row);                     // position of this lane's query column
-  const int pos_max = ctx - (q_end - (row0 + n_rows - 1));
+  const int pos_min = ctx - (q_end - row0), pos_max = pos_min + n_rows - 1;
   const int KD = a.maps * a.dim;
   const int kc = (a.dim + 15) >> 4, vt = (a.vdim + 15) >> 4;
+  const bool vec_k = a.vec_k && (a.dim & 3) == 0;
   const T* qrow = static_cast<const T*>(a.q) + (static_cast<size_t>(row) * a.H + h) * KD;
-  const bool vec_q = (KD & 3) == 0 && a.vec_k;
 
   F qf[2][KC];
 #pragma unroll
@@ -65,7 +234,7 @@ __global__ __launch_bounds__(256) void prefill_kernel(AttnArgs a) {
 #pragma unroll
     for (int c = 0; c < KC; ++c) {
       const int f = 16 * c + 4 * grp;
-      qf[m][c] = (m < a.maps && c < kc) ? load_frag<T>(qrow + m * a.dim + f, a.dim - f, vec_q && (a.dim & 3) == 0) : zero_frag<T>();
+      qf[m][c] = (m < a.maps && c < kc) ? load_frag_t<T, FULL>(qrow + m * a.dim + f, a.dim - f, vec_k) : zero_frag<T>();
     }
   f32x4 acc[2][VT];
 #pragma unroll
@@ -73,73 +242,8 @@ __global__ __launch_bounds__(256) void prefill_kernel(AttnArgs a) {
 #pragma unroll
     for (int t = 0; t < VT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   float mx[2] = {-INFINITY, -INFINITY}, den[2] = {0.f, 0.f};
-  const int* table = a.block_tables + static_cast<size_t>(seq) * a.max_blocks;
-  const T* kc_base = static_cast<const T*>(a.k_cache);
-  const T* vc_base = static_cast<const T*>(a.v_cache);
-
-  for (int kb = 0; 16 * kb <= pos_max; ++kb) {
-    const int key0 = 16 * kb;
-    int page = table[key0 / a.BS];
-    page = (page < 0 || page >= a.num_blocks) ? 0 : page;
-    const int koff = key0 % a.BS;
-    // ---- S^T = K Q^T: A = K rows (key col, features 4 grp + j) ----
-    const T* krow = kc_base + ((static_cast<size_t>(page) * a.G + g) * a.BS + koff + col) * KD;
-    f32x4 s[2];
-#pragma unroll
-    for (int m = 0; m < 2; ++m) {
-      s[m] = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (m < a.maps) {
-#pragma unroll
-        for (int c = 0; c < KC; ++c)
-          if (c < kc) {
-            const int f = 16 * c + 4 * grp;
-            const F kf = load_frag<T>(krow + m * a.dim + f, a.dim - f, a.vec_k && (a.dim & 3) == 0);
-            s[m] = mma16(kf, qf[m][c], s[m]);
-          }
-      }
-    }
-    // ---- online softmax per query column; lane holds keys key0 + 4 grp + i ----
-    F pf[2];
-#pragma unroll
-    for (int m = 0; m < 2; ++m) {
-      if (m >= a.maps) { pf[m] = zero_frag<T>(); continue; }
-      float v[4], bm = -INFINITY;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        v[i] = (key0 + 4 * grp + i <= pos) ? s[m][i] * a.scale : -INFINITY;
-        bm = fmaxf(bm, v[i]);
-      }
-      bm = fmaxf(bm, __shfl_xor(bm, 16, WAVE));
-      bm = fmaxf(bm, __shfl_xor(bm, 32, WAVE));
-      const float m_new = fmaxf(mx[m], bm);               // finite: key 0 is visible to every query
-      const float alpha = expf(mx[m] - m_new);
-      float ps = 0.f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        v[i] = expf(v[i] - m_new);
-        ps += v[i];
-      }
-      ps += __shfl_xor(ps, 16, WAVE);
-      ps += __shfl_xor(ps, 32, WAVE);
-      den[m] = den[m] * alpha + ps;
-      mx[m] = m_new;
-#pragma unroll
-      for (int t = 0; t < VT; ++t)
-        if (t < vt) acc[m][t] *= alpha;
-      pf[m] = Elem<T>::pack(v[0], v[1], v[2], v[3]);
-    }
-    // ---- O^T += V^T P^T: A = V^T rows (feature 16 t + col, keys 4 grp + j) ----
-#pragma unroll
-    for (int t = 0; t < VT; ++t)
-      if (t < vt) {
-        const int e = 16 * t + col;
-        F vf = zero_frag<T>();
-        if (e < a.vdim)
-          vf = load_frag<T>(vc_base + ((static_cast<size_t>(page) * a.G + g) * a.vdim + e) * a.BS + koff + 4 * grp, 4, a.vec_v);
-        acc[0][t] = mma16(vf, pf[0], acc[0][t]);
-        if (a.maps > 1) acc[1][t] = mma16(vf, pf[1], acc[1][t]);
-      }
-  }
+  attend_range<T, KC, VT, KT, PF, FULL>(a, g, qf, pos, pos_min, 0, pos_max,
+                                        a.block_tables + static_cast<size_t>(seq) * a.max_blocks, acc, mx, den);
   // ---- combine the maps, unit norm over the head's value features, store ----
   const float i0 = 1.0f / den[0], i1 = a.maps > 1 ? a.lam / den[1] : 0.f;
   float ss = 0.f;
@@ -171,109 +275,65 @@ __global__ __launch_bounds__(256) void prefill_kernel(AttnArgs a) {
   }
 }
 
-// ws layout per (item, head, split): [maps] max, [maps] denominator, [maps][vdim] numerators.
-template <typename T, int VPL>
-__global__ __launch_bounds__(64) void decode_kernel(AttnArgs a, int n_items) {
-  extern __shared__ float smem[];
-  const int lane = threadIdx.x;
-  const int h = blockIdx.x, split = blockIdx.y, item = blockIdx.z;
-  const int g = h / (a.H / a.G);
+// Single-token rows, the query heads of one KV head packed into the 16 MFMA columns: column c is
+// head g (H / G) + 16 cg + c of the same token, so K and V^T are read once per KV head.  One wave
+// per (item, KV head x column group, SPLIT_KEYS-key split); partials as the merge kernel reads them
+// (running maxima in the log2 domain of `attend_range`).
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL>
+__global__ __launch_bounds__(64) void decode_mfma_kernel(AttnArgs a) {
+  typedef typename Elem<T>::frag F;
+  const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
+  const int per = a.H / a.G;
+  const int g = blockIdx.x % a.G, cg = blockIdx.x / a.G;
+  const int split = blockIdx.y, item = blockIdx.z;
   const int row = a.work ? a.work[2 * item] : item, seq = a.work ? a.work[2 * item + 1] : item;
   const int ctx = a.seq_lens[seq];
   const int k_begin = split * SPLIT_KEYS, k_end = min(ctx, k_begin + SPLIT_KEYS);
   if (k_begin >= k_end) return;
+  const bool col_ok = 16 * cg + col < per;
+  const int h = g * per + min(16 * cg + col, per - 1);
   const int KD = a.maps * a.dim;
-  float* qs = smem;                  // [KD] scaled query
-  float* ps = smem + KD;             // [maps][64] probabilities of the chunk
+  const int kc = (a.dim + 15) >> 4, vt = (a.vdim + 15) >> 4;
+  const bool vec_k = a.vec_k && (a.dim & 3) == 0;
   const T* qrow = static_cast<const T*>(a.q) + (static_cast<size_t>(row) * a.H + h) * KD;
-  for (int i = lane; i < KD; i += 64) qs[i] = Elem<T>::ld(qrow[i]) * a.scale;
-  __syncthreads();
-  const int* table = a.block_tables + static_cast<size_t>(seq) * a.max_blocks;
-  const T* kc_base = static_cast<const T*>(a.k_cache);
-  const T* vc_base = static_cast<const T*>(a.v_cache);
-  float mx[2] = {-INFINITY, -INFINITY}, den[2] = {0.f, 0.f};
-  float acc[2][VPL];
+  F qf[2][KC];
 #pragma unroll
   for (int m = 0; m < 2; ++m)
 #pragma unroll
-    for (int j = 0; j < VPL; ++j) acc[m][j] = 0.f;
-
-  for (int c0 = k_begin; c0 < k_end; c0 += 64) {
-    const int key = c0 + lane;
-    const bool ok = key < k_end;
-    float s[2] = {-INFINITY, -INFINITY};
-    if (ok) {
-      int page = table[key / a.BS];
-      page = (page < 0 || page >= a.num_blocks) ? 0 : page;
-      const T* krow = kc_base + ((static_cast<size_t>(page) * a.G + g) * a.BS + key % a.BS) * KD;
-      for (int m = 0; m < a.maps; ++m) {
-        float d = 0.f;
-        const T* kp = krow + m * a.dim;
-        const float* qp = qs + m * a.dim;
-        if (a.vec_k && (a.dim & 3) == 0) {
-          for (int f = 0; f < a.dim; f += 4) {
-            const typename Elem<T>::frag kv = *reinterpret_cast<const typename Elem<T>::frag*>(kp + f);
+    for (int c = 0; c < KC; ++c) {
+      const int f = 16 * c + 4 * grp;
+      qf[m][c] = (m < a.maps && c < kc) ? load_frag_t<T, FULL>(qrow + m * a.dim + f, a.dim - f, vec_k) : zero_frag<T>();
+    }
+  f32x4 acc[2][VT];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              float kvj;
-              if constexpr (sizeof(T) == 2) kvj = bf2f(static_cast<bf16_t>(kv[j])); else kvj = kv[j];
-              d += qp[f + j] * kvj;
-            }
-          }
-        } else {
-          for (int f = 0; f < a.dim; ++f) d += qp[f] * Elem<T>::ld(kp[f]);
-        }
-        s[m] = d;
-      }
-    }
-    __syncthreads();  // the previous chunk's probabilities have been read
-    float alpha[2] = {1.f, 1.f};
-    for (int m = 0; m < a.maps; ++m) {
-      const float m_new = fmaxf(mx[m], wave_max(s[m]));   // finite: the chunk holds >= 1 key
-      alpha[m] = expf(mx[m] - m_new);
-      const float p = ok ? expf(s[m] - m_new) : 0.f;
-      den[m] = den[m] * alpha[m] + wave_sum(p);
-      mx[m] = m_new;
-      ps[m * 64 + lane] = p;
-    }
-    __syncthreads();
-    // ---- values: this lane owns features lane + 64 j; 16 contiguous keys per page group ----
-    const int n_grp = (min(64, k_end - c0) + 15) >> 4;
+  for (int m = 0; m < 2; ++m)
 #pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      const int e = lane + 64 * j;
-      if (e < a.vdim) {
-        float a0 = 0.f, a1 = 0.f;
-        for (int gi = 0; gi < n_grp; ++gi) {
-          const int key0 = c0 + 16 * gi;
-          int page = table[key0 / a.BS];
-          page = (page < 0 || page >= a.num_blocks) ? 0 : page;
-          const T* vp = vc_base + ((static_cast<size_t>(page) * a.G + g) * a.vdim + e) * a.BS + key0 % a.BS;
-          const int n_ok = min(16, k_end - key0);
-          for (int kk = 0; kk < n_ok; ++kk) {     // (keys past the end hold stale data: never read)
-            const float v = Elem<T>::ld(vp[kk]);
-            a0 += ps[16 * gi + kk] * v;
-            if (a.maps > 1) a1 += ps[64 + 16 * gi + kk] * v;
-          }
-        }
-        acc[0][j] = acc[0][j] * alpha[0] + a0;
-        acc[1][j] = acc[1][j] * alpha[1] + a1;
-      }
-    }
-  }
+    for (int t = 0; t < VT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float mx[2] = {-INFINITY, -INFINITY}, den[2] = {0.f, 0.f};
+  attend_range<T, KC, VT, KT, PF, FULL>(a, g, qf, k_end - 1, k_end - 1, k_begin, k_end - 1,
+                                        a.block_tables + static_cast<size_t>(seq) * a.max_blocks, acc, mx, den);
+  if (!col_ok) return;
   float* w = a.ws + ((static_cast<size_t>(item) * a.H + h) * a.n_splits + split) * (2 * a.maps + a.maps * a.vdim);
-  if (lane < a.maps) {
-    w[lane] = mx[lane];
-    w[a.maps + lane] = den[lane];
-  }
-  for (int m = 0; m < a.maps; ++m)
 #pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      const int e = lane + 64 * j;
-      if (e < a.vdim) w[2 * a.maps + m * a.vdim + e] = acc[m][j];
+  for (int m = 0; m < 2; ++m)
+    if (grp == 0 && m < a.maps) {
+      w[m] = mx[m];
+      w[a.maps + m] = den[m];
     }
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int t = 0; t < VT; ++t)
+      if (m < a.maps && t < vt) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int e = 16 * t + 4 * grp + i;
+          if (e < a.vdim) w[2 * a.maps + m * a.vdim + e] = acc[m][t][i];
+        }
+      }
 }
 
+// ws layout per (item, head, split): [maps] max, [maps] denominator, [maps][vdim] numerators.
 template <typename T, int VPL>
 __global__ __launch_bounds__(64) void decode_merge_kernel(AttnArgs a) {
   const int lane = threadIdx.x, h = blockIdx.x, item = blockIdx.y;
@@ -292,7 +352,7 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(AttnArgs a) {
 #pragma unroll
     for (int j = 0; j < VPL; ++j) num[j] = 0.f;
     for (int s = 0; s < n; ++s) {
-      const float f = expf(w[s * stride + m] - mx);
+      const float f = exp2f(w[s * stride + m] - mx);   // (maxima are kept in the log2 domain)
       den += w[s * stride + a.maps + m] * f;
 #pragma unroll
       for (int j = 0; j < VPL; ++j) {
@@ -318,24 +378,39 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(AttnArgs a) {
 }
 
 template <typename T>
-int launch_prefill(const AttnArgs& a, int n_tiles, hipStream_t s) {
+int launch_prefill(const AttnArgs& a, int n_tiles, int tile_rows, hipStream_t s) {
   dim3 grid(n_tiles, a.H);
-  if (a.dim <= 64 && a.vdim <= 128) prefill_kernel<T, 4, 8><<<grid, 256, 0, s>>>(a);
-  else prefill_kernel<T, 8, 16><<<grid, 256, 0, s>>>(a);
+  const bool small = a.dim <= 64 && a.vdim <= 128;
+  const bool full = a.dim % 16 == 0 && a.vdim % 16 == 0 && a.vec_k && a.vec_v;   // whole, aligned fragments only
+  if (tile_rows != 64) return -2;
+  if (small && sizeof(T) == 2) {
+    if (full) prefill_kernel<T, 4, 8, 2, true, true><<<grid, 256, 0, s>>>(a);
+    else prefill_kernel<T, 4, 8, 2, true, false><<<grid, 256, 0, s>>>(a);
+  } else if (small) {
+    if (full) prefill_kernel<T, 4, 8, 1, false, true><<<grid, 256, 0, s>>>(a);
+    else prefill_kernel<T, 4, 8, 1, false, false><<<grid, 256, 0, s>>>(a);
+  } else {   // (the branch-free form of the wide instance runs out of registers)
+    prefill_kernel<T, 8, 16, 1, false, false><<<grid, 256, 0, s>>>(a);
+  }
   return BCG_CHECK_LAUNCH();
 }
 
 template <typename T>
 int launch_decode(const AttnArgs& a, int n_items, hipStream_t s) {
-  dim3 grid(a.H, a.n_splits, n_items);
-  const size_t lds = sizeof(float) * (a.maps * a.dim + 2 * 64);
-  if (a.vdim <= 128) {
-    decode_kernel<T, 2><<<grid, 64, lds, s>>>(a, n_items);
-    decode_merge_kernel<T, 2><<<dim3(a.H, n_items), 64, 0, s>>>(a);
+  const int per = a.H / a.G;
+  dim3 grid(a.G * ((per + 15) / 16), a.n_splits, n_items);
+  const bool full = a.dim % 16 == 0 && a.vdim % 16 == 0 && a.vec_k && a.vec_v;
+  if (a.dim <= 64 && a.vdim <= 128 && sizeof(T) == 2) {
+    if (full) decode_mfma_kernel<T, 4, 8, 2, true, true><<<grid, 64, 0, s>>>(a);
+    else decode_mfma_kernel<T, 4, 8, 2, true, false><<<grid, 64, 0, s>>>(a);
+  } else if (a.dim <= 64 && a.vdim <= 128) {
+    if (full) decode_mfma_kernel<T, 4, 8, 1, false, true><<<grid, 64, 0, s>>>(a);
+    else decode_mfma_kernel<T, 4, 8, 1, false, false><<<grid, 64, 0, s>>>(a);
   } else {
-    decode_kernel<T, 4><<<grid, 64, lds, s>>>(a, n_items);
-    decode_merge_kernel<T, 4><<<dim3(a.H, n_items), 64, 0, s>>>(a);
+    decode_mfma_kernel<T, 8, 16, 1, false, false><<<grid, 64, 0, s>>>(a);
   }
+  if (a.vdim <= 128) decode_merge_kernel<T, 2><<<dim3(a.H, n_items), 64, 0, s>>>(a);
+  else decode_merge_kernel<T, 4><<<dim3(a.H, n_items), 64, 0, s>>>(a);
   return BCG_CHECK_LAUNCH();
 }
 
@@ -349,7 +424,7 @@ BCG_API int bcg_multimap_attention(int mode, const void* q, const void* k_cache,
                                    const void* block_tables, int max_blocks, const void* q_start, const void* seq_lens,
                                    const void* work, int n_work, void* out, void* ws, int n_splits, int H, int G, int maps,
                                    int dim, int vdim, int BS, int num_blocks, float scale, float lam, float head_eps,
-                                   float out_scale, int is_f32, void* stream) {
+                                   float out_scale, int tile_rows, int is_f32, void* stream) {
   if (n_work <= 0) return 0;
   if (maps < 1 || maps > 2 || dim > 128 || vdim > 256 || BS % 16 || H % G || n_work > 65535 * 16) return -2;
   AttnArgs a;
@@ -362,8 +437,9 @@ BCG_API int bcg_multimap_attention(int mode, const void* q, const void* k_cache,
   a.scale = scale; a.lam = lam; a.head_eps = head_eps; a.out_scale = out_scale;
   a.vec_k = ((maps * dim) % 4 == 0) ? 1 : 0;
   a.vec_v = 1;  // BS % 16 == 0: every 4-key group of a V^T row is aligned
+  a.swz = a.vec_k;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (mode == 0) return is_f32 ? launch_prefill<float>(a, n_work, s) : launch_prefill<bf16_t>(a, n_work, s);
+  if (mode == 0) return is_f32 ? launch_prefill<float>(a, n_work, tile_rows, s) : launch_prefill<bf16_t>(a, n_work, tile_rows, s);
   if (n_splits < 1 || H > 65535 || n_splits > 65535 || n_work > 65535) return -2;
   return is_f32 ? launch_decode<float>(a, n_work, s) : launch_decode<bf16_t>(a, n_work, s);
 }

@@ -11,11 +11,13 @@ template <> struct Elem<bf16_t> {
   typedef s16x4 frag;  // 4 consecutive elements: one lane's share of a 16-deep MFMA operand
   static __device__ __forceinline__ float ld(bf16_t v) { return bf2f(v); }
   static __device__ __forceinline__ bf16_t st(float f) { return f2bf(f); }
+  // finite inputs (softmax weights): the hardware's round-to-nearest-even conversion
   static __device__ __forceinline__ frag pack(float a, float b, float c, float d) {
-    frag r;
-    r[0] = static_cast<short>(f2bf(a)); r[1] = static_cast<short>(f2bf(b));
-    r[2] = static_cast<short>(f2bf(c)); r[3] = static_cast<short>(f2bf(d));
-    return r;
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+    bf16x4 r;
+    r[0] = static_cast<__bf16>(a); r[1] = static_cast<__bf16>(b);
+    r[2] = static_cast<__bf16>(c); r[3] = static_cast<__bf16>(d);
+    return __builtin_bit_cast(frag, r);
   }
 };
 template <> struct Elem<float> {
@@ -55,6 +57,14 @@ __device__ __forceinline__ typename Elem<T>::frag load_frag(const T* p, int n_va
     if constexpr (sizeof(T) == 2) r[j] = static_cast<short>(v); else r[j] = v;
   }
   return r;
+}
+
+// FULL: the caller guarantees four valid, vector-aligned elements (no branch around the load,
+// so a run of fragment loads is issued back to back).
+template <typename T, bool FULL>
+__device__ __forceinline__ typename Elem<T>::frag load_frag_t(const T* p, int n_valid, bool vec) {
+  if constexpr (FULL) return *reinterpret_cast<const typename Elem<T>::frag*>(p);
+  else return load_frag<T>(p, n_valid, vec);
 }
 
 template <typename T>

@@ -14,7 +14,7 @@
 
 namespace {
 
-constexpr int TM = 32, TN = 128, MAX_E = 256;
+constexpr int TM = 64, TN = 256, MAX_E = 256;  // position tile rows, output columns per workgroup (4 waves x 64)
 
 template <typename T>
 __global__ __launch_bounds__(64) void route_kernel(const T* __restrict__ h, const float* __restrict__ rw,
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(1024) void align_kernel(const int* __restrict__ idx
 
 // Position p of tile blockIdx.x: slot = sorted[p] (-1: padding).  gather: A row = a[(slot / top)]
 // (token rows), else a[p].  scatter: output row = slot, else p.  act 1: relu squared.
-template <typename T>
+template <typename T, bool FULL>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w,
                                                        T* __restrict__ out, int64_t out_stride,
                                                        const int* __restrict__ sorted,
@@ -99,15 +99,15 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, 
   if (e < 0) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
-  const int p0 = blockIdx.x * TM, n0 = blockIdx.y * TN + 32 * wave;
+  const int p0 = blockIdx.x * TM, n0 = blockIdx.y * TN + 64 * wave;   // a wave: all 64 rows x 64 columns
   if (n0 >= N) return;
   const T* we = w + static_cast<size_t>(e) * N * K;
-  const T* arow[2];
-  int slot[2];
-  const T* wrow[2];
-  bool wok[2];
+  const T* arow[4];
+  int slot[4];
+  const T* wrow[4];
+  bool wok[4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < 4; ++i) {
     const int p = p0 + 16 * i + col;
     slot[i] = sorted[p];
     const int64_t r = gather ? (slot[i] < 0 ? 0 : slot[i] / top) : p;
@@ -116,29 +116,30 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, 
     wok[i] = n < N;
     wrow[i] = we + static_cast<size_t>(wok[i] ? n : 0) * K;
   }
-  f32x4 acc[2][2];  // [n tile][m tile]: lane holds C[m = col][n = 4 grp + i]
+  f32x4 acc[4][4];  // [n tile][m tile]: lane holds C[m = col][n = 4 grp + i]
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
   for (int k = 4 * grp; k < K; k += 16) {
-    F af[2], wf[2];
+    F af[4], wf[4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      af[i] = slot[i] >= 0 ? load_frag<T>(arow[i] + k, K - k, vec) : zero_frag<T>();
-      wf[i] = wok[i] ? load_frag<T>(wrow[i] + k, K - k, vec) : zero_frag<T>();
+    for (int i = 0; i < 4; ++i) {
+      af[i] = slot[i] >= 0 ? load_frag_t<T, FULL>(arow[i] + k, K - k, vec) : zero_frag<T>();
+      wf[i] = wok[i] ? load_frag_t<T, FULL>(wrow[i] + k, K - k, vec) : zero_frag<T>();
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = mma16(wf[i], af[j], acc[i][j]);
+      for (int j = 0; j < 4; ++j) acc[i][j] = mma16(wf[i], af[j], acc[i][j]);
   }
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < 4; ++j) {
     if (slot[j] < 0) continue;
     const int64_t r = scatter ? slot[j] : p0 + 16 * j + col;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int n = n0 + 16 * i + 4 * grp + q;
@@ -201,14 +202,17 @@ BCG_API int bcg_moe_gemm(const void* a, int64_t a_stride, const void* w, void* o
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(n_tiles, (N + TN - 1) / TN);
   const int vec = (K % 4 == 0 && a_stride % 4 == 0) ? 1 : 0;
-  if (is_f32)
-    moe_gemm_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(a), a_stride, static_cast<const float*>(w),
-                                               static_cast<float*>(out), out_stride, static_cast<const int*>(sorted),
-                                               static_cast<const int*>(tile_expert), N, K, top, gather, scatter, act, vec);
-  else
-    moe_gemm_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(a), a_stride, static_cast<const bf16_t*>(w),
-                                                static_cast<bf16_t*>(out), out_stride, static_cast<const int*>(sorted),
-                                                static_cast<const int*>(tile_expert), N, K, top, gather, scatter, act, vec);
+#define BCG_MOE_GEMM(TYPE, FULL_)                                                                                    \
+  moe_gemm_kernel<TYPE, FULL_><<<grid, 256, 0, s>>>(static_cast<const TYPE*>(a), a_stride, static_cast<const TYPE*>(w), \
+                                                    static_cast<TYPE*>(out), out_stride, static_cast<const int*>(sorted), \
+                                                    static_cast<const int*>(tile_expert), N, K, top, gather, scatter, act, vec)
+  const bool full = vec && K % 16 == 0;   // whole, aligned fragments only
+  if (is_f32) {
+    if (full) BCG_MOE_GEMM(float, true); else BCG_MOE_GEMM(float, false);
+  } else {
+    if (full) BCG_MOE_GEMM(bf16_t, true); else BCG_MOE_GEMM(bf16_t, false);
+  }
+#undef BCG_MOE_GEMM
   return BCG_CHECK_LAUNCH();
 }
 

@@ -94,7 +94,8 @@ __global__ __launch_bounds__(NT) void act_kernel(const T* __restrict__ in, T* __
 
 // One block per token.  Row layout [q (n_q maps dim) | k (n_kv maps dim) | v (n_kv vdim) | ...].
 // Feature i < 2 half of every map pairs with i +- half; angle = position * inv_freq[i % half] (fp32).
-// K -> k_cache [NB, n_kv, BS, maps dim], V -> v_cache [NB, n_kv, vdim, BS] at `slots[t]`.
+// K -> k_cache [NB, n_kv, BS, maps dim], V -> v_cache [NB, n_kv, vdim, BS] at `slots[t]` (slabs
+// stored fragment-major when maps dim is a multiple of 4: see seqmix_attention.hip).
 template <typename T>
 __global__ __launch_bounds__(NT) void rope_multi_kv_kernel(const T* __restrict__ qkv, int64_t row_stride,
                                                            const int* __restrict__ positions,
@@ -124,14 +125,21 @@ __global__ __launch_bounds__(NT) void rope_multi_kv_kernel(const T* __restrict__
       q_out[static_cast<size_t>(t) * qw + idx] = Elem<T>::st(val);
     } else if (kv_ok) {
       const int kk = idx - qw;
-      const int g = kk / (maps * dim), f = kk - g * maps * dim;
-      k_cache[((static_cast<size_t>(blk) * n_kv + g) * BS + off) * (maps * dim) + f] = Elem<T>::st(val);
+      const int KD = maps * dim;
+      const int g = kk / KD, f = kk - g * KD;
+      T* slab = k_cache + (static_cast<size_t>(blk) * n_kv + g) * BS * KD;
+      // KD % 4 == 0: fragment-major slab [KD / 4][BS][4] (seqmix_attention.hip); else [BS][KD]
+      if ((KD & 3) == 0) slab[(static_cast<size_t>(f >> 2) * BS + off) * 4 + (f & 3)] = Elem<T>::st(val);
+      else slab[static_cast<size_t>(off) * KD + f] = Elem<T>::st(val);
     }
   }
   if (kv_ok) {
     for (int idx = threadIdx.x; idx < vw; idx += NT) {
       const int g = idx / vdim, e = idx - g * vdim;
-      v_cache[((static_cast<size_t>(blk) * n_kv + g) * vdim + e) * BS + off] = row[qw + kw + idx];
+      T* slab = v_cache + (static_cast<size_t>(blk) * n_kv + g) * vdim * BS;
+      // fragment-major slab [BS / 4][vdim][4] with the K rule above; else [vdim][BS]
+      if (((maps * dim) & 3) == 0) slab[(static_cast<size_t>(off >> 2) * vdim + e) * 4 + (off & 3)] = row[qw + kw + idx];
+      else slab[static_cast<size_t>(e) * BS + off] = row[qw + kw + idx];
     }
   }
 }

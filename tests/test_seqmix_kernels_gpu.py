@@ -58,7 +58,7 @@ def test_act_fn_strided(ops, dtype, kind):
     torch.testing.assert_close(ops.act_fn(view, kind).float(), ref.act_fn(view, kind).float(), **_tol(dtype))
 
 
-def _paged(seq_lens, q_lens, BS, G, KD, VD, dtype, seed, shuffle=True):
+def _paged(seq_lens, q_lens, BS, G, KD, VD, dtype, seed, shuffle=True, tile_rows=64):
     """Random paged cache + metadata of a packed step: sequence b holds seq_lens[b] tokens, the last q_lens[b] are queries."""
     g = torch.Generator().manual_seed(seed)
     nblk = [(n + BS - 1) // BS for n in seq_lens]
@@ -77,12 +77,12 @@ def _paged(seq_lens, q_lens, BS, G, KD, VD, dtype, seed, shuffle=True):
         if ql == 1:
             single.append((q_start[-1], b))
         else:
-            for t in range(q_start[-1], q_start[-1] + ql, 64):
-                tiles.append((b, t, min(t + 64, q_start[-1] + ql)))
+            for t in range(q_start[-1], q_start[-1] + ql, tile_rows):
+                tiles.append((b, t, min(t + tile_rows, q_start[-1] + ql)))
         q_start.append(q_start[-1] + ql)
     i32 = torch.int32
     meta = AttnMeta(positions=None, slots=None, block_tables=bt.to(DEV), seq_lens=torch.tensor(seq_lens, dtype=i32, device=DEV),
-                    q_start=torch.tensor(q_start, dtype=i32, device=DEV), decode=False,
+                    q_start=torch.tensor(q_start, dtype=i32, device=DEV), decode=False, tile_rows=tile_rows,
                     tiles=torch.tensor(tiles, dtype=i32, device=DEV).reshape(-1, 3),
                     single=torch.tensor(single, dtype=i32, device=DEV).reshape(-1, 2))
     return k.to(DEV), v.to(DEV), meta, q_start[-1]
@@ -92,19 +92,21 @@ def _paged(seq_lens, q_lens, BS, G, KD, VD, dtype, seed, shuffle=True):
 @pytest.mark.parametrize("H,G,maps,dim,vdim,BS", [(4, 2, 2, 32, 64, 16), (3, 3, 2, 24, 40, 16), (4, 1, 1, 64, 128, 32),
                                                  (2, 2, 2, 80, 144, 16), (2, 1, 2, 20, 18, 16)])
 def test_multimap_attention_mixed_step(ops, dtype, H, G, maps, dim, vdim, BS):
-    seq_lens = [300, 17, 1, 129, 64, 513, 40]
-    q_lens = [70, 17, 1, 1, 2, 1, 16]
-    k, v, meta, T = _paged(seq_lens, q_lens, BS, G, maps * dim, vdim, dtype, seed=dim)
+    seq_lens = [300, 17, 1, 129, 64, 513, 40, 400]
+    q_lens = [70, 17, 1, 1, 2, 1, 16, 301]
+    k, v, meta, T = _paged(seq_lens, q_lens, BS, G, maps * dim, vdim, dtype, seed=dim,
+                           tile_rows=ops.multimap_tile_rows(dim, vdim))
     q = torch.randn(T, H, maps * dim, generator=torch.Generator().manual_seed(1)).to(dtype).to(DEV)
     args = (0.17, maps, 0.35, 1e-5, 0.4, vdim)
-    got = ops.multimap_attention(q, k, v, meta, *args)
+    kp, vp = ops.kv_from_logical(k, v)   # the kernels' slab order
+    got = ops.multimap_attention(q, kp, vp, meta, *args)
     want = ref.multimap_attention(q, k, v, meta.block_tables, meta.q_start, meta.seq_lens, *args)
     torch.testing.assert_close(got.float(), want.float(), **(dict(atol=3e-2, rtol=3e-2) if dtype == torch.bfloat16 else dict(atol=1e-4, rtol=1e-4)))
     # the same rows through the decode form of a step: every sequence one token
     B = len(seq_lens)
     dmeta = AttnMeta(positions=None, slots=None, block_tables=meta.block_tables, seq_lens=meta.seq_lens, decode=True)
     qd = q[(meta.q_start[1:] - 1).long()].contiguous()
-    got_d = ops.multimap_attention(qd, k, v, dmeta, *args)
+    got_d = ops.multimap_attention(qd, kp, vp, dmeta, *args)
     want_d = ref.multimap_attention(qd, k, v, meta.block_tables, torch.arange(B + 1, dtype=torch.int32, device=DEV),
                                     meta.seq_lens, *args)
     torch.testing.assert_close(got_d.float(), want_d.float(), **(dict(atol=3e-2, rtol=3e-2) if dtype == torch.bfloat16 else dict(atol=1e-4, rtol=1e-4)))
@@ -123,7 +125,7 @@ def test_attention_far_key_stands_out(ops, dtype):
         blk2 = int(meta.block_tables[b, (far + 300) // BS])
         k[blk2, 0, (far + 300) % BS, dim:] = 6.0 * q[0 if b == 0 else T - 1, 0, dim:]
     args = (0.2, maps, 0.5, 1e-5, 1.0, vdim)
-    got = ops.multimap_attention(q, k, v, meta, *args)
+    got = ops.multimap_attention(q, *ops.kv_from_logical(k, v), meta, *args)
     want = ref.multimap_attention(q, k, v, meta.block_tables, meta.q_start, meta.seq_lens, *args)
     torch.testing.assert_close(got.float(), want.float(), **(dict(atol=3e-2, rtol=3e-2) if dtype == torch.bfloat16 else dict(atol=1e-4, rtol=1e-4)))
 
@@ -144,8 +146,9 @@ def test_rope_multi_kv_write(ops, dtype, n_q, n_kv, maps, dim, vdim, rot):
     q_r = ref.rope_multi_kv_write(qkv, pos, slots, n_q, n_kv, maps, dim, vdim, inv, *caches[1])
     tol = dict(atol=3e-2, rtol=2e-2) if dtype == torch.bfloat16 else dict(atol=2e-3, rtol=1e-3)  # fp32 sin/cos at large angles
     torch.testing.assert_close(q.float(), q_r.float(), **tol)
-    torch.testing.assert_close(caches[0][0].float(), caches[1][0].float(), **tol)
-    torch.testing.assert_close(caches[0][1].float(), caches[1][1].float(), atol=0, rtol=0)
+    k_l, v_l = ops.kv_to_logical(*caches[0])
+    torch.testing.assert_close(k_l.float(), caches[1][0].float(), **tol)
+    torch.testing.assert_close(v_l.float(), caches[1][1].float(), atol=0, rtol=0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
