@@ -52,8 +52,8 @@ struct AttnArgs {
 // columns of a wave (column = a query row of one head, or a query head of one token).
 //   limit      per lane: the last key its column may see;  limit_min: the smallest over the wave
 //   KT         16-key tiles per iteration (one softmax update and one rescale per iteration)
-//   PF         the next iteration's K fragments are loaded before this iteration's products and
-//              this iteration's V^T fragments before its QK^T products (loads fly under the MFMAs)
+//   PF         this iteration's V^T fragments are loaded before its QK^T products and the next
+//              iteration's K fragments right after them (loads fly under the MFMAs and the softmax)
 //   FULL       whole, aligned fragments only (no branch around any load)
 // Everything that does not depend on the lane stays scalar: the page lookup and the slab base go
 // to SGPRs, a lane adds a 32-bit offset that is fixed for the whole loop.  Scores are kept in the
@@ -69,20 +69,12 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a, int g, const typ
   const int kc = (a.dim + 15) >> 4, vt = (a.vdim + 15) >> 4;
   const bool vec_k = a.vec_k && (a.dim & 3) == 0;
   const float sc = a.scale * 1.4426950408889634f;
-  // lane offsets inside a (page, KV head) slab; the slab base and the key offset are wave-uniform
-  uint32_t koffs[2][KC], voffs[VT];
-#pragma unroll
-  for (int m = 0; m < 2; ++m)
-#pragma unroll
-    for (int c = 0; c < KC; ++c) {
-      const int f = 16 * c + 4 * grp;        // this lane: key col, features m dim + f .. + 3
-      koffs[m][c] = a.swz ? (((m * a.dim + f) >> 2) * a.BS + col) * 4 : col * KD + m * a.dim + f;
-    }
-#pragma unroll
-  for (int t = 0; t < VT; ++t) {
-    const int e = 16 * t + col;              // this lane: value feature e, keys 4 grp .. + 3
-    voffs[t] = a.swz ? (grp * a.vdim + e) * 4 : e * a.BS + 4 * grp;
-  }
+  // offsets inside a (page, KV head) slab = one lane offset (fixed for the whole loop) + a
+  // wave-uniform offset per fragment; the slab base and the tile's key offset are uniform too
+  const uint32_t k_lane = a.swz ? (grp * a.BS + col) * 4 : col * KD + 4 * grp;
+  const uint32_t v_lane = a.swz ? (grp * a.vdim + col) * 4 : col * a.BS + 4 * grp;
+  auto k_uni = [&](int m, int c) { return a.swz ? ((m * a.dim + 16 * c) >> 2) * a.BS * 4 : m * a.dim + 16 * c; };
+  auto v_uni = [&](int t) { return a.swz ? 16 * t * 4 : 16 * t * a.BS; };
   const int k_mul = a.swz ? 4 : KD, v_mul = a.swz ? a.vdim : 1;   // slab offset per key of the tile's first key
   const T* kc_base = static_cast<const T*>(a.k_cache);
   const T* vc_base = static_cast<const T*>(a.v_cache);
@@ -107,35 +99,25 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a, int g, const typ
       for (int m = 0; m < 2; ++m)
 #pragma unroll
         for (int c = 0; c < KC; ++c)
-          kf[u][m][c] = (m < a.maps && c < kc) ? load_frag_t<T, FULL>(kp + koffs[m][c], a.dim - (16 * c + 4 * grp), vec_k)
+          kf[u][m][c] = (m < a.maps && c < kc) ? load_frag_t<T, FULL>(kp + k_uni(m, c) + k_lane, a.dim - (16 * c + 4 * grp), vec_k)
                                                : zero_frag<T>();
     }
   };
 
-  F kn[KT][2][KC];
-  if (PF) load_k(k_begin, kn);
+  F kf[KT][2][KC];
+  if (PF) load_k(k_begin, kf);
   for (int key0 = k_begin; key0 <= k_last; key0 += 16 * KT) {
     F vf[PF ? KT : 1][PF ? VT : 1];
     auto load_v = [&](int u, int t) {
       const T *kp, *vp;
       slabs(key0 + 16 * u, kp, vp);
-      return (t < vt && 16 * t + col < a.vdim) ? load_frag_t<T, FULL>(vp + voffs[t], 4, a.vec_v) : zero_frag<T>();
+      return (t < vt && 16 * t + col < a.vdim) ? load_frag_t<T, FULL>(vp + v_uni(t) + v_lane, 4, a.vec_v) : zero_frag<T>();
     };
     if constexpr (PF) {
 #pragma unroll
       for (int u = 0; u < KT; ++u)
 #pragma unroll
         for (int t = 0; t < VT; ++t) vf[u][t] = load_v(u, t);
-    }
-    F kf[KT][2][KC];
-    if (PF) {
-#pragma unroll
-      for (int u = 0; u < KT; ++u)
-#pragma unroll
-        for (int m = 0; m < 2; ++m)
-#pragma unroll
-          for (int c = 0; c < KC; ++c) kf[u][m][c] = kn[u][m][c];
-      if (key0 + 16 * KT <= k_last) load_k(key0 + 16 * KT, kn);
     } else {
       load_k(key0, kf);
     }
@@ -152,6 +134,9 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a, int g, const typ
             if (c < kc) s[u][m] = mma16(kf[u][m][c], qf[m][c], s[u][m]);
         }
       }
+    // the K fragments are spent: the next iteration's go into the same registers, under the
+    // softmax and the second product
+    if (PF && key0 + 16 * KT <= k_last) load_k(key0 + 16 * KT, kf);
     // ---- online softmax per query column; lane holds keys key0 + 16 u + 4 grp + i ----
     const bool masked = key0 + 16 * KT - 1 > limit_min;     // (wave-uniform) some key of the iteration is hidden
     F pf[KT][2];
@@ -210,8 +195,8 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a, int g, const typ
   }
 }
 
-template <typename T, int KC, int VT, int KT, bool PF, bool FULL>
-__global__ __launch_bounds__(256) void prefill_kernel(AttnArgs a) {
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC>
+__global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
   typedef typename Elem<T>::frag F;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col = lane & 15, grp = lane >> 4;
@@ -279,8 +264,8 @@ __global__ __launch_bounds__(256) void prefill_kernel(AttnArgs a) {
 // head g (H / G) + 16 cg + c of the same token, so K and V^T are read once per KV head.  One wave
 // per (item, KV head x column group, SPLIT_KEYS-key split); partials as the merge kernel reads them
 // (running maxima in the log2 domain of `attend_range`).
-template <typename T, int KC, int VT, int KT, bool PF, bool FULL>
-__global__ __launch_bounds__(64) void decode_mfma_kernel(AttnArgs a) {
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC>
+__global__ __launch_bounds__(64, OCC) void decode_mfma_kernel(AttnArgs a) {
   typedef typename Elem<T>::frag F;
   const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
   const int per = a.H / a.G;
@@ -383,14 +368,16 @@ int launch_prefill(const AttnArgs& a, int n_tiles, int tile_rows, hipStream_t s)
   const bool small = a.dim <= 64 && a.vdim <= 128;
   const bool full = a.dim % 16 == 0 && a.vdim % 16 == 0 && a.vec_k && a.vec_v;   // whole, aligned fragments only
   if (tile_rows != 64) return -2;
-  if (small && sizeof(T) == 2) {
-    if (full) prefill_kernel<T, 4, 8, 2, true, true><<<grid, 256, 0, s>>>(a);
-    else prefill_kernel<T, 4, 8, 2, true, false><<<grid, 256, 0, s>>>(a);
-  } else if (small) {
-    if (full) prefill_kernel<T, 4, 8, 1, false, true><<<grid, 256, 0, s>>>(a);
-    else prefill_kernel<T, 4, 8, 1, false, false><<<grid, 256, 0, s>>>(a);
+  if constexpr (sizeof(T) == 2) if (small) {
+    if (full) prefill_kernel<T, 4, 8, 2, true, true, 2><<<grid, 256, 0, s>>>(a);
+    else prefill_kernel<T, 4, 8, 2, true, false, 2><<<grid, 256, 0, s>>>(a);
+    return BCG_CHECK_LAUNCH();
+  }
+  if (small) {
+    if (full) prefill_kernel<T, 4, 8, 1, false, true, 2><<<grid, 256, 0, s>>>(a);
+    else prefill_kernel<T, 4, 8, 1, false, false, 2><<<grid, 256, 0, s>>>(a);
   } else {   // (the branch-free form of the wide instance runs out of registers)
-    prefill_kernel<T, 8, 16, 1, false, false><<<grid, 256, 0, s>>>(a);
+    prefill_kernel<T, 8, 16, 1, false, false, 1><<<grid, 256, 0, s>>>(a);
   }
   return BCG_CHECK_LAUNCH();
 }
@@ -400,14 +387,18 @@ int launch_decode(const AttnArgs& a, int n_items, hipStream_t s) {
   const int per = a.H / a.G;
   dim3 grid(a.G * ((per + 15) / 16), a.n_splits, n_items);
   const bool full = a.dim % 16 == 0 && a.vdim % 16 == 0 && a.vec_k && a.vec_v;
-  if (a.dim <= 64 && a.vdim <= 128 && sizeof(T) == 2) {
-    if (full) decode_mfma_kernel<T, 4, 8, 2, true, true><<<grid, 64, 0, s>>>(a);
-    else decode_mfma_kernel<T, 4, 8, 2, true, false><<<grid, 64, 0, s>>>(a);
+  bool done = false;
+  if constexpr (sizeof(T) == 2) if (a.dim <= 64 && a.vdim <= 128) {
+    done = true;
+    if (full) decode_mfma_kernel<T, 4, 8, 2, true, true, 2><<<grid, 64, 0, s>>>(a);
+    else decode_mfma_kernel<T, 4, 8, 2, true, false, 2><<<grid, 64, 0, s>>>(a);
+  }
+  if (done) {
   } else if (a.dim <= 64 && a.vdim <= 128) {
-    if (full) decode_mfma_kernel<T, 4, 8, 1, false, true><<<grid, 64, 0, s>>>(a);
-    else decode_mfma_kernel<T, 4, 8, 1, false, false><<<grid, 64, 0, s>>>(a);
+    if (full) decode_mfma_kernel<T, 4, 8, 1, false, true, 2><<<grid, 64, 0, s>>>(a);
+    else decode_mfma_kernel<T, 4, 8, 1, false, false, 2><<<grid, 64, 0, s>>>(a);
   } else {
-    decode_mfma_kernel<T, 8, 16, 1, false, false><<<grid, 64, 0, s>>>(a);
+    decode_mfma_kernel<T, 8, 16, 1, false, false, 1><<<grid, 64, 0, s>>>(a);
   }
   if (a.vdim <= 128) decode_merge_kernel<T, 2><<<dim3(a.H, n_items), 64, 0, s>>>(a);
   else decode_merge_kernel<T, 4><<<dim3(a.H, n_items), 64, 0, s>>>(a);

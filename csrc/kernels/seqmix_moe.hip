@@ -152,6 +152,117 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, 
   }
 }
 
+// The same product with both operands staged through LDS (K a multiple of 32, 16-byte aligned
+// rows): a workgroup loads its 64 x 32 slice of A and 256 x 32 slice of W_e with 16-byte row-wise
+// loads (the next slice is in flight in registers while the current one is multiplied), and the
+// waves read their MFMA fragments from LDS (rows padded by 8 elements).  bf16 uses the 32-deep
+// v_mfma_f32_16x16x32_bf16 (a lane holds 8 consecutive k of its row), fp32 the 4-deep fp32 MFMA.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gemm_lds_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w,
+                                                           T* __restrict__ out, int64_t out_stride,
+                                                           const int* __restrict__ sorted,
+                                                           const int* __restrict__ tile_expert, int N, int K, int top,
+                                                           int gather, int scatter, int act) {
+  typedef typename Elem<T>::frag F;
+  constexpr int BK = 32, LDK = BK + 8;   // rows stay 16-byte aligned for the 8-element fragment reads
+  typedef T Chunk __attribute__((ext_vector_type(8)));   // 8 consecutive elements (16 or 32 bytes)
+  __shared__ __attribute__((aligned(16))) T As[TM * LDK];
+  __shared__ __attribute__((aligned(16))) T Ws[TN * LDK];
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int p0 = blockIdx.x * TM, nb = blockIdx.y * TN;
+  const T* we = w + static_cast<size_t>(e) * N * K;
+  // staging role: row tid / 4 of the slice, 8 elements at k = 8 (tid % 4)
+  const int s_row = tid >> 2, s_k = (tid & 3) * 8;
+  const int a_slot = sorted[p0 + s_row];
+  const T* a_src = a + (gather ? static_cast<int64_t>(a_slot < 0 ? 0 : a_slot / top) : static_cast<int64_t>(p0 + s_row)) * a_stride + s_k;
+  const T* w_src[4];
+  bool w_ok[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = nb + s_row + 64 * i;
+    w_ok[i] = n < N;
+    w_src[i] = we + static_cast<size_t>(w_ok[i] ? n : 0) * K + s_k;
+  }
+  Chunk ra, rw0, rw1, rw2, rw3;
+  auto get = [&](const T* p, bool ok) {
+    Chunk c = Chunk(T(0));
+    if (ok) c = *reinterpret_cast<const Chunk*>(p);
+    return c;
+  };
+  auto fetch = [&](int k0) {
+    ra = get(a_src + k0, a_slot >= 0);
+    rw0 = get(w_src[0] + k0, w_ok[0]);
+    rw1 = get(w_src[1] + k0, w_ok[1]);
+    rw2 = get(w_src[2] + k0, w_ok[2]);
+    rw3 = get(w_src[3] + k0, w_ok[3]);
+  };
+  int slot[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) slot[j] = sorted[p0 + 16 * j + col];
+  f32x4 acc[4][4];  // [n tile][m tile]: lane holds C[m = col][n = 4 grp + i]
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    __syncthreads();   // the previous slice has been read
+    *reinterpret_cast<Chunk*>(&As[s_row * LDK + s_k]) = ra;
+    *reinterpret_cast<Chunk*>(&Ws[(s_row + 0) * LDK + s_k]) = rw0;
+    *reinterpret_cast<Chunk*>(&Ws[(s_row + 64) * LDK + s_k]) = rw1;
+    *reinterpret_cast<Chunk*>(&Ws[(s_row + 128) * LDK + s_k]) = rw2;
+    *reinterpret_cast<Chunk*>(&Ws[(s_row + 192) * LDK + s_k]) = rw3;
+    __syncthreads();
+    if (k0 + BK < K) fetch(k0 + BK);
+    if constexpr (sizeof(T) == 2) {
+      bf16x8 af[4], wf[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        af[i] = *reinterpret_cast<const bf16x8*>(&As[(16 * i + col) * LDK + 8 * grp]);
+        wf[i] = *reinterpret_cast<const bf16x8*>(&Ws[(64 * wave + 16 * i + col) * LDK + 8 * grp]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], af[j], acc[i][j], 0, 0, 0);
+    } else {
+#pragma unroll
+    for (int ks = 0; ks < BK; ks += 16) {
+      F af[4], wf[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        af[i] = *reinterpret_cast<const F*>(&As[(16 * i + col) * LDK + ks + 4 * grp]);
+        wf[i] = *reinterpret_cast<const F*>(&Ws[(64 * wave + 16 * i + col) * LDK + ks + 4 * grp]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = mma16(wf[i], af[j], acc[i][j]);
+    }
+    }
+  }
+  const int n0 = nb + 64 * wave;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (slot[j] < 0) continue;
+    const int64_t r = scatter ? slot[j] : p0 + 16 * j + col;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + 16 * i + 4 * grp + q;
+        if (n < N) {
+          float v = acc[i][j][q];
+          if (act == 1) { v = fmaxf(v, 0.f); v *= v; }
+          out[r * out_stride + n] = Elem<T>::st(v);
+        }
+      }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ y, const float* __restrict__ wts,
                                                       float* __restrict__ out, int W, int top) {
@@ -207,6 +318,18 @@ BCG_API int bcg_moe_gemm(const void* a, int64_t a_stride, const void* w, void* o
                                                     static_cast<TYPE*>(out), out_stride, static_cast<const int*>(sorted), \
                                                     static_cast<const int*>(tile_expert), N, K, top, gather, scatter, act, vec)
   const bool full = vec && K % 16 == 0;   // whole, aligned fragments only
+  const int esz = is_f32 ? 4 : 2;
+  if (K % 32 == 0 && (a_stride * esz) % 16 == 0 && (reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(w)) % 16 == 0) {
+    if (is_f32)
+      moe_gemm_lds_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(a), a_stride, static_cast<const float*>(w),
+                                                     static_cast<float*>(out), out_stride, static_cast<const int*>(sorted),
+                                                     static_cast<const int*>(tile_expert), N, K, top, gather, scatter, act);
+    else
+      moe_gemm_lds_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(a), a_stride, static_cast<const bf16_t*>(w),
+                                                      static_cast<bf16_t*>(out), out_stride, static_cast<const int*>(sorted),
+                                                      static_cast<const int*>(tile_expert), N, K, top, gather, scatter, act);
+    return BCG_CHECK_LAUNCH();
+  }
   if (is_f32) {
     if (full) BCG_MOE_GEMM(float, true); else BCG_MOE_GEMM(float, false);
   } else {

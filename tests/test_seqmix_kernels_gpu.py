@@ -152,7 +152,8 @@ def test_rope_multi_kv_write(ops, dtype, n_q, n_kv, maps, dim, vdim, rot):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,W,E,top,ff", [(1, 64, 4, 1, 32), (5, 128, 8, 2, 48), (333, 256, 6, 3, 100), (64, 96, 3, 3, 36)])
+@pytest.mark.parametrize("T,W,E,top,ff", [(1, 64, 4, 1, 32), (5, 128, 8, 2, 48), (333, 256, 6, 3, 100), (64, 96, 3, 3, 36),
+                                          (700, 512, 8, 2, 320), (130, 72, 5, 2, 40)])
 def test_moe_route_and_experts(ops, dtype, T, W, E, top, ff):
     g = torch.Generator().manual_seed(T + E)
     h = torch.randn(T, W, generator=g).to(dtype).to(DEV)
