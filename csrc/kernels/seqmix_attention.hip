@@ -58,15 +58,25 @@ struct AttnArgs {
 // Everything that does not depend on the lane stays scalar: the page lookup and the slab base go
 // to SGPRs, a lane adds a 32-bit offset that is fixed for the whole loop.  Scores are kept in the
 // log2 domain (scale * log2 e folded into one multiply, v_exp_f32 directly).
-template <typename T, int KC, int VT, int KT, bool PF, bool FULL>
-__device__ __forceinline__ void attend_range(const AttnArgs& a, int g, const typename Elem<T>::frag (&qf)[2][KC],
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL, bool EXACT>
+__device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const typename Elem<T>::frag (&qf)[2][KC],
                                              int limit, int limit_min, int k_begin, int k_last,
                                              const int* __restrict__ table, f32x4 (&acc)[2][VT], float (&mx)[2],
                                              float (&den)[2]) {
   typedef typename Elem<T>::frag F;
+  // EXACT: two maps, dim = 16 KC, vdim = 16 VT, 16-token pages, fragment-major slabs -- every guard
+  // below is a compile-time constant, fragment offsets are immediates, the loop body is straight-line
+  struct Shape {
+    const AttnArgs& r;
+    int maps, dim, vdim, swz, BS, G, max_blocks, num_blocks, vec_k, vec_v;
+    float scale;
+    const void *k_cache, *v_cache;
+  };
+  const Shape a{a_, EXACT ? 2 : a_.maps, EXACT ? 16 * KC : a_.dim, EXACT ? 16 * VT : a_.vdim, EXACT ? 1 : a_.swz, EXACT ? 16 : a_.BS, a_.G,
+                a_.max_blocks, a_.num_blocks, EXACT ? 1 : a_.vec_k, EXACT ? 1 : a_.vec_v, a_.scale, a_.k_cache, a_.v_cache};
   const int lane = threadIdx.x & 63, col = lane & 15, grp = lane >> 4;
   const int KD = a.maps * a.dim;
-  const int kc = (a.dim + 15) >> 4, vt = (a.vdim + 15) >> 4;
+  const int kc = EXACT ? KC : (a.dim + 15) >> 4, vt = EXACT ? VT : (a.vdim + 15) >> 4;
   const bool vec_k = a.vec_k && (a.dim & 3) == 0;
   const float sc = a.scale * 1.4426950408889634f;
   // offsets inside a (page, KV head) slab = one lane offset (fixed for the whole loop) + a
@@ -80,38 +90,49 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a, int g, const typ
   const T* vc_base = static_cast<const T*>(a.v_cache);
   const size_t k_slab = static_cast<size_t>(a.BS) * KD, v_slab = static_cast<size_t>(a.BS) * a.vdim;
 
-  // tiles past the sequence read some valid page: every one of their keys is masked
-  auto slabs = [&](int key0, const T*& kp, const T*& vp) {
-    const int idx = min(key0 / a.BS, a.max_blocks - 1);
-    int page = table[idx];
-    page = (page < 0 || page >= a.num_blocks) ? 0 : page;
-    const size_t base = static_cast<size_t>(page) * a.G + g;
-    const int koff = key0 - (key0 / a.BS) * a.BS;
-    kp = kc_base + base * k_slab + koff * k_mul;
-    vp = vc_base + base * v_slab + koff * v_mul;
+  // A cursor walks the sequence in 16-key tiles: page index + key offset in the page, stepped
+  // without a division (BS is a multiple of 16).  Tiles past the sequence read some valid page:
+  // every one of their keys is masked.
+  struct Cursor { int p, o; };
+  auto step = [&](Cursor& c) {
+    c.o += 16;
+    if (c.o >= a.BS) { c.o = 0; ++c.p; }
   };
-  auto load_k = [&](int key0, F (&kf)[KT][2][KC]) {
+  auto slab_base = [&](const Cursor& c) {
+    int page = table[min(c.p, a.max_blocks - 1)];
+    page = (page < 0 || page >= a.num_blocks) ? 0 : page;
+    return static_cast<size_t>(page) * a.G + g;
+  };
+  auto load_k = [&](Cursor& c, F (&kf)[KT][2][KC]) {
 #pragma unroll
     for (int u = 0; u < KT; ++u) {
-      const T *kp, *vp;
-      slabs(key0 + 16 * u, kp, vp);
+      const T* kp = kc_base + slab_base(c) * k_slab + c.o * k_mul;
+      step(c);
 #pragma unroll
       for (int m = 0; m < 2; ++m)
 #pragma unroll
-        for (int c = 0; c < KC; ++c)
-          kf[u][m][c] = (m < a.maps && c < kc) ? load_frag_t<T, FULL>(kp + k_uni(m, c) + k_lane, a.dim - (16 * c + 4 * grp), vec_k)
-                                               : zero_frag<T>();
+        for (int c2 = 0; c2 < KC; ++c2)
+          kf[u][m][c2] = (m < a.maps && c2 < kc) ? load_frag_t<T, FULL>(kp + k_uni(m, c2) + k_lane, a.dim - (16 * c2 + 4 * grp), vec_k)
+                                                 : zero_frag<T>();
     }
   };
 
+  Cursor k_cur, v_cur;
+  k_cur.p = k_begin / a.BS;
+  k_cur.o = k_begin - k_cur.p * a.BS;
+  v_cur = k_cur;
   F kf[KT][2][KC];
-  if (PF) load_k(k_begin, kf);
+  if (PF) load_k(k_cur, kf);
   for (int key0 = k_begin; key0 <= k_last; key0 += 16 * KT) {
+    const T* vps[KT];
+#pragma unroll
+    for (int u = 0; u < KT; ++u) {
+      vps[u] = vc_base + slab_base(v_cur) * v_slab + v_cur.o * v_mul;
+      step(v_cur);
+    }
     F vf[PF ? KT : 1][PF ? VT : 1];
     auto load_v = [&](int u, int t) {
-      const T *kp, *vp;
-      slabs(key0 + 16 * u, kp, vp);
-      return (t < vt && 16 * t + col < a.vdim) ? load_frag_t<T, FULL>(vp + v_uni(t) + v_lane, 4, a.vec_v) : zero_frag<T>();
+      return (t < vt && 16 * t + col < a.vdim) ? load_frag_t<T, FULL>(vps[u] + v_uni(t) + v_lane, 4, a.vec_v) : zero_frag<T>();
     };
     if constexpr (PF) {
 #pragma unroll
@@ -119,7 +140,7 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a, int g, const typ
 #pragma unroll
         for (int t = 0; t < VT; ++t) vf[u][t] = load_v(u, t);
     } else {
-      load_k(key0, kf);
+      load_k(k_cur, kf);
     }
     // ---- S^T = K Q^T ----
     f32x4 s[KT][2];
@@ -136,7 +157,7 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a, int g, const typ
       }
     // the K fragments are spent: the next iteration's go into the same registers, under the
     // softmax and the second product
-    if (PF && key0 + 16 * KT <= k_last) load_k(key0 + 16 * KT, kf);
+    if (PF && key0 + 16 * KT <= k_last) load_k(k_cur, kf);
     // ---- online softmax per query column; lane holds keys key0 + 16 u + 4 grp + i ----
     const bool masked = key0 + 16 * KT - 1 > limit_min;     // (wave-uniform) some key of the iteration is hidden
     F pf[KT][2];
@@ -195,7 +216,7 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a, int g, const typ
   }
 }
 
-template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC>
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC, bool EXACT = false>
 __global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
   typedef typename Elem<T>::frag F;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -227,7 +248,7 @@ __global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
 #pragma unroll
     for (int t = 0; t < VT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   float mx[2] = {-INFINITY, -INFINITY}, den[2] = {0.f, 0.f};
-  attend_range<T, KC, VT, KT, PF, FULL>(a, g, qf, pos, pos_min, 0, pos_max,
+  attend_range<T, KC, VT, KT, PF, FULL, EXACT>(a, g, qf, pos, pos_min, 0, pos_max,
                                         a.block_tables + static_cast<size_t>(seq) * a.max_blocks, acc, mx, den);
   // ---- combine the maps, unit norm over the head's value features, store ----
   const float i0 = 1.0f / den[0], i1 = a.maps > 1 ? a.lam / den[1] : 0.f;
@@ -264,7 +285,7 @@ __global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
 // head g (H / G) + 16 cg + c of the same token, so K and V^T are read once per KV head.  One wave
 // per (item, KV head x column group, SPLIT_KEYS-key split); partials as the merge kernel reads them
 // (running maxima in the log2 domain of `attend_range`).
-template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC>
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC, bool EXACT = false>
 __global__ __launch_bounds__(64, OCC) void decode_mfma_kernel(AttnArgs a) {
   typedef typename Elem<T>::frag F;
   const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
@@ -295,7 +316,7 @@ __global__ __launch_bounds__(64, OCC) void decode_mfma_kernel(AttnArgs a) {
 #pragma unroll
     for (int t = 0; t < VT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   float mx[2] = {-INFINITY, -INFINITY}, den[2] = {0.f, 0.f};
-  attend_range<T, KC, VT, KT, PF, FULL>(a, g, qf, k_end - 1, k_end - 1, k_begin, k_end - 1,
+  attend_range<T, KC, VT, KT, PF, FULL, EXACT>(a, g, qf, k_end - 1, k_end - 1, k_begin, k_end - 1,
                                         a.block_tables + static_cast<size_t>(seq) * a.max_blocks, acc, mx, den);
   if (!col_ok) return;
   float* w = a.ws + ((static_cast<size_t>(item) * a.H + h) * a.n_splits + split) * (2 * a.maps + a.maps * a.vdim);
@@ -369,6 +390,14 @@ int launch_prefill(const AttnArgs& a, int n_tiles, int tile_rows, hipStream_t s)
   const bool full = a.dim % 16 == 0 && a.vdim % 16 == 0 && a.vec_k && a.vec_v;   // whole, aligned fragments only
   if (tile_rows != 64) return -2;
   if constexpr (sizeof(T) == 2) if (small) {
+    const bool exact = full && a.maps == 2 && a.swz && a.BS == 16;
+#define BCG_EXACT(KC_, VT_)                                                                      \
+  if (exact && a.dim == 16 * KC_ && a.vdim == 16 * VT_) {                                        \
+    prefill_kernel<T, KC_, VT_, 2, true, true, 2, true><<<grid, 256, 0, s>>>(a);                 \
+    return BCG_CHECK_LAUNCH();                                                                   \
+  }
+    BCG_EXACT(4, 8) BCG_EXACT(3, 6) BCG_EXACT(2, 4) BCG_EXACT(4, 4) BCG_EXACT(2, 2)
+#undef BCG_EXACT
     if (full) prefill_kernel<T, 4, 8, 2, true, true, 2><<<grid, 256, 0, s>>>(a);
     else prefill_kernel<T, 4, 8, 2, true, false, 2><<<grid, 256, 0, s>>>(a);
     return BCG_CHECK_LAUNCH();
@@ -390,6 +419,17 @@ int launch_decode(const AttnArgs& a, int n_items, hipStream_t s) {
   bool done = false;
   if constexpr (sizeof(T) == 2) if (a.dim <= 64 && a.vdim <= 128) {
     done = true;
+    const bool exact = full && a.maps == 2 && a.swz && a.BS == 16;
+    bool hit = false;
+#define BCG_EXACT(KC_, VT_)                                                                      \
+  if (!hit && exact && a.dim == 16 * KC_ && a.vdim == 16 * VT_) {                                \
+    hit = true;                                                                                  \
+    decode_mfma_kernel<T, KC_, VT_, 2, true, true, 2, true><<<grid, 64, 0, s>>>(a);              \
+  }
+    BCG_EXACT(4, 8) BCG_EXACT(3, 6) BCG_EXACT(2, 4) BCG_EXACT(4, 4) BCG_EXACT(2, 2)
+#undef BCG_EXACT
+    if (hit) {
+    } else
     if (full) decode_mfma_kernel<T, 4, 8, 2, true, true, 2><<<grid, 64, 0, s>>>(a);
     else decode_mfma_kernel<T, 4, 8, 2, true, false, 2><<<grid, 64, 0, s>>>(a);
   }

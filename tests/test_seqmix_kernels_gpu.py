@@ -90,7 +90,8 @@ def _paged(seq_lens, q_lens, BS, G, KD, VD, dtype, seed, shuffle=True, tile_rows
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,maps,dim,vdim,BS", [(4, 2, 2, 32, 64, 16), (3, 3, 2, 24, 40, 16), (4, 1, 1, 64, 128, 32),
-                                                 (2, 2, 2, 80, 144, 16), (2, 1, 2, 20, 18, 16)])
+                                                 (2, 2, 2, 80, 144, 16), (2, 1, 2, 20, 18, 16), (8, 2, 2, 64, 128, 16),
+                                                 (6, 2, 2, 48, 96, 16), (2, 2, 2, 64, 64, 16), (40, 2, 2, 32, 32, 16)])
 def test_multimap_attention_mixed_step(ops, dtype, H, G, maps, dim, vdim, BS):
     seq_lens = [300, 17, 1, 129, 64, 513, 40, 400]
     q_lens = [70, 17, 1, 1, 2, 1, 16, 301]
@@ -139,7 +140,7 @@ def test_rope_multi_kv_write(ops, dtype, n_q, n_kv, maps, dim, vdim, rot):
     qkv = torch.randn(T, width, generator=g).to(dtype).to(DEV)
     pos = torch.randint(0, 5000, (T,), generator=g, dtype=torch.int32).to(DEV)
     slots = (torch.randperm((NB - 1) * BS, generator=g)[:T] + BS).to(torch.int32).to(DEV)
-    inv = ref.rope_inv_freq(rot, 250000.0, DEV)
+    inv = ref.rope_inv_freq(rot, 30000.0, DEV)
     caches = [[torch.zeros(NB, n_kv, BS, maps * dim, dtype=dtype, device=DEV),
                torch.zeros(NB, n_kv, vdim, BS, dtype=dtype, device=DEV)] for _ in range(2)]
     q = ops.rope_multi_kv_write(qkv, pos, slots, n_q, n_kv, maps, dim, vdim, inv, *caches[0])
