@@ -16,28 +16,36 @@ namespace {
 
 constexpr int TM = 64, TN = 256, MAX_E = 256;  // position tile rows, output columns per workgroup (4 waves x 64)
 
+// One workgroup per token: the four waves share the experts (and the gate row), a wave's lanes
+// stride over the width with 16-byte loads of the fp32 router rows; thread 0 then picks the top-k.
 template <typename T>
-__global__ __launch_bounds__(64) void route_kernel(const T* __restrict__ h, const float* __restrict__ rw,
-                                                   const float* __restrict__ rb, const float* __restrict__ gw,
-                                                   int* __restrict__ idx, float* __restrict__ wts,
-                                                   float* __restrict__ gate, int W, int E, int top) {
-  __shared__ float z[MAX_E];
-  const int t = blockIdx.x, lane = threadIdx.x;
+__global__ __launch_bounds__(256) void route_kernel(const T* __restrict__ h, const float* __restrict__ rw,
+                                                    const float* __restrict__ rb, const float* __restrict__ gw,
+                                                    int* __restrict__ idx, float* __restrict__ wts,
+                                                    float* __restrict__ gate, int W, int E, int top) {
+  __shared__ float z[MAX_E + 1];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* row = h + static_cast<size_t>(t) * W;
-  for (int e = 0; e < E; ++e) {
+  const int rows = E + (gw != nullptr ? 1 : 0);
+  const bool vec = (W & 3) == 0;
+  for (int e = wave; e < rows; e += 4) {
+    const float* wrow = e < E ? rw + static_cast<size_t>(e) * W : gw;
     float d = 0.f;
-    for (int i = lane; i < W; i += 64) d += Elem<T>::ld(row[i]) * rw[static_cast<size_t>(e) * W + i];
+    if (vec) {
+      for (int i = 4 * lane; i < W; i += 256) {
+        const f32x4 wv = *reinterpret_cast<const f32x4*>(wrow + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) d += Elem<T>::ld(row[i + j]) * wv[j];
+      }
+    } else {
+      for (int i = lane; i < W; i += 64) d += Elem<T>::ld(row[i]) * wrow[i];
+    }
     d = wave_sum(d);
-    if (lane == 0) z[e] = d + (rb ? rb[e] : 0.f);
-  }
-  if (gw != nullptr) {
-    float d = 0.f;
-    for (int i = lane; i < W; i += 64) d += Elem<T>::ld(row[i]) * gw[i];
-    d = wave_sum(d);
-    if (lane == 0) gate[t] = d;
+    if (lane == 0) z[e] = d + ((e < E && rb) ? rb[e] : 0.f);
   }
   __syncthreads();
-  if (lane == 0) {
+  if (threadIdx.x == 0) {
+    if (gw != nullptr) gate[t] = z[E];
     float best0 = 0.f, den = 0.f;
     for (int j = 0; j < top; ++j) {
       int be = 0;
@@ -284,11 +292,11 @@ BCG_API int bcg_moe_route(const void* h, const void* rw, const void* rb, const v
   if (E < 1 || E > MAX_E || top < 1 || top > E) return -2;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (is_f32)
-    route_kernel<float><<<T_, 64, 0, s>>>(static_cast<const float*>(h), static_cast<const float*>(rw), static_cast<const float*>(rb),
+    route_kernel<float><<<T_, 256, 0, s>>>(static_cast<const float*>(h), static_cast<const float*>(rw), static_cast<const float*>(rb),
                                          static_cast<const float*>(gw), static_cast<int*>(idx), static_cast<float*>(wts),
                                          static_cast<float*>(gate), W, E, top);
   else
-    route_kernel<bf16_t><<<T_, 64, 0, s>>>(static_cast<const bf16_t*>(h), static_cast<const float*>(rw), static_cast<const float*>(rb),
+    route_kernel<bf16_t><<<T_, 256, 0, s>>>(static_cast<const bf16_t*>(h), static_cast<const float*>(rw), static_cast<const float*>(rb),
                                           static_cast<const float*>(gw), static_cast<int*>(idx), static_cast<float*>(wts),
                                           static_cast<float*>(gate), W, E, top);
   return BCG_CHECK_LAUNCH();
