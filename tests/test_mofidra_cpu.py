@@ -286,3 +286,25 @@ def test_text_entry_point_with_id_prompts(tmp_path):
         assert len(ids) == 5 and ids[0] == int(O.forward(cfg, sd, prompt)[-1].argmax())
     finally:
         llm.shutdown()
+
+
+def test_generate_command_line(tmp_path, capsys):
+    from byzantine_consensus_llm_agents_amd.engine.generate import main
+    cfg = C.CASES["plain"]
+    path = str(tmp_path / "m")
+    sd = _f64(C.checkpoint(cfg, path, seed=6))
+    prompts = [C.tokens(7, cfg["vocab"], 1), C.tokens(20, cfg["vocab"], 2)]
+    argv = ["--weights", path, "--backend", "torch", "--dtype", "float32", "--max-tokens", "3", "--max-model-len", "64"]
+    for p in prompts:
+        argv += ["--prompt", " ".join(map(str, p))]
+    assert main(argv) == 0
+    lines = [l for l in capsys.readouterr().out.strip().splitlines() if l.strip()]
+    assert len(lines) == 2
+    for p, line in zip(prompts, lines):
+        ids = [int(t) for t in line.split()]
+        assert len(ids) == 3 and ids[0] == int(O.forward(cfg, sd, p)[-1].argmax())
+
+
+def test_bench_option_leaves_the_default_workload():
+    import bench
+    assert bench.parse([]).family_compare is False and bench.parse(["--family-compare"]).family_compare is True
