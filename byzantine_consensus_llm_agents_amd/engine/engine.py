@@ -443,29 +443,41 @@ class InferenceEngine:
         bs = self.args.kv_block_size
         wave, chunk, want = [], [], []
         with self._device_ctx():
+            # check the whole step before anything changes: a refused step leaves every stream as it was
+            free_rows = sum(1 for r in self.slots if r is None)
+            need_blocks, seen = 0, set()
+            for sid, tokens, w in entries:
+                if sid in seen:
+                    raise ValueError(f"stream {sid!r} appears twice in one step")
+                seen.add(sid)
+                req = self._streams.get(sid)
+                have = len(req.seq.prompt_ids) if req is not None else 0
+                held = len(req.seq.blocks) if req is not None else 0
+                if not tokens or have + len(tokens) > self.args.max_model_len:
+                    raise ValueError("stream entry empty or beyond max_model_len")
+                if any(not 0 <= int(o) < len(tokens) for o in w):
+                    raise ValueError("wanted offset outside the entry")
+                free_rows -= req is None
+                need_blocks += max(0, (have + len(tokens) + bs - 1) // bs - held)
+            if free_rows < 0:
+                raise RuntimeError("no free state row for a new stream")
+            if need_blocks > self.blocks.num_free_blocks:
+                raise RuntimeError("KV pool exhausted")
             for sid, tokens, w in entries:
                 req = self._streams.get(sid)
                 if req is None:
-                    free = [i for i, r in enumerate(self.slots) if r is None]
-                    if not free:
-                        raise RuntimeError("no free state row for a new stream")
                     req = _Request(_Seq(0, [], 0, 0.0, None))
-                    req.row, req.pending = free[0], True
+                    req.row, req.pending = self.slots.index(None), True
                     self.slots[req.row] = self._streams[sid] = req
                 seq = req.seq
                 a = len(seq.prompt_ids)
-                if not tokens or a + len(tokens) > self.args.max_model_len:
-                    raise ValueError("stream entry empty or beyond max_model_len")
                 need = (a + len(tokens) + bs - 1) // bs - len(seq.blocks)
                 if need > 0:
-                    more = self.blocks.grow(need)
-                    if not more:
-                        raise RuntimeError("KV pool exhausted")
-                    seq.blocks.extend(more)
+                    seq.blocks.extend(self.blocks.grow(need))
                 seq.prompt_ids.extend(int(t) for t in tokens)
                 chunk.append((len(wave), a, a + len(tokens)))
                 wave.append(seq)
-                want.append(list(w))
+                want.append([int(o) for o in w])
             logits = None
             if chunk:
                 table_cpu = self._block_table(wave, len(wave))

@@ -249,10 +249,12 @@ def test_long_decoding(case):
 def test_pool_exhaustion_is_an_error_not_a_wrong_answer(case):
     cfg, sd, eng = case
     free = eng.blocks.num_free_blocks
-    eng.stream_step([("w", C.tokens(100, cfg["vocab"], 7), [])])
-    with pytest.raises(RuntimeError):
-        eng.stream_step([("x", C.tokens(16 * free - 50, cfg["vocab"], 7), [])])
-    eng.stream_step([], end=["x", "w"])
+    toks = C.tokens(100, cfg["vocab"], 7)
+    eng.stream_step([("w", toks[:60], [])])
+    with pytest.raises(RuntimeError):   # refused as a whole: "w" keeps its 60 tokens, "x" never opens
+        eng.stream_step([("w", toks[60:70], [0]), ("x", C.tokens(16 * free - 50, cfg["vocab"], 7), [])])
+    assert "x" not in eng._streams and len(eng._streams["w"].seq.prompt_ids) == 60
+    _close(eng.stream_step([("w", toks[60:], [39])], end=["w"]), _oracle(cfg, sd, toks)[99:100])
     assert eng.blocks.num_free_blocks == free and not any(eng.slots)
 
 
