@@ -91,7 +91,8 @@ def _paged(seq_lens, q_lens, BS, G, KD, VD, dtype, seed, shuffle=True, tile_rows
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,maps,dim,vdim,BS", [(4, 2, 2, 32, 64, 16), (3, 3, 2, 24, 40, 16), (4, 1, 1, 64, 128, 32),
                                                  (2, 2, 2, 80, 144, 16), (2, 1, 2, 20, 18, 16), (8, 2, 2, 64, 128, 16),
-                                                 (6, 2, 2, 48, 96, 16), (2, 2, 2, 64, 64, 16), (40, 2, 2, 32, 32, 16)])
+                                                 (6, 2, 2, 48, 96, 16), (2, 2, 2, 64, 64, 16), (40, 2, 2, 32, 32, 16), (2, 1, 2, 9, 10, 16),
+                                                 (3, 1, 1, 7, 5, 16)])
 def test_multimap_attention_mixed_step(ops, dtype, H, G, maps, dim, vdim, BS):
     seq_lens = [300, 17, 1, 129, 64, 513, 40, 400]
     q_lens = [70, 17, 1, 1, 2, 1, 16, 301]
@@ -132,7 +133,8 @@ def test_attention_far_key_stands_out(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("n_q,n_kv,maps,dim,vdim,rot", [(4, 2, 2, 32, 64, 32), (3, 1, 2, 24, 20, 8), (2, 2, 1, 64, 64, 0)])
+@pytest.mark.parametrize("n_q,n_kv,maps,dim,vdim,rot", [(4, 2, 2, 32, 64, 32), (3, 1, 2, 24, 20, 8), (2, 2, 1, 64, 64, 0),
+                                                        (2, 1, 2, 9, 10, 4)])
 def test_rope_multi_kv_write(ops, dtype, n_q, n_kv, maps, dim, vdim, rot):
     T, BS, NB = 45, 16, 9
     g = torch.Generator().manual_seed(rot)
