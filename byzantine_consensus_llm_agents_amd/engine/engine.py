@@ -163,6 +163,7 @@ class _Seq:
     done_pos: int = 0               # prompt tokens whose KV is written (prefix cache + prefilled chunks)
     error: Optional[str] = None
     max_new_requested: int = 0      # the caller's max_tokens (before the context-room clamp)
+    row: int = -1                   # the request's state row (models with per-sequence state)
 
 
 class InferenceEngine:
@@ -198,7 +199,7 @@ class InferenceEngine:
         self.ops = get_ops(self.backend)
 
         model_dir = args.weights if args.weights not in ("random", "auto") else None
-        if model_dir and not os.path.exists(os.path.join(model_dir, "tokenizer.json")) and cfg.family == "mofidra":
+        if model_dir and not os.path.exists(os.path.join(model_dir, "tokenizer.json")) and cfg.family in ("mofidra", "padadra"):
             from .tokenizer import IdTokenizer
             self.tokenizer = IdTokenizer(cfg.vocab_size)  # a checkpoint of weights only: prompts are token ids
         else:
@@ -283,7 +284,7 @@ class InferenceEngine:
         a, m = self.args, self.model
         bs = a.kv_block_size
         kv_dtype = self.kv_dtype()
-        per_block = m.kv_block_bytes(bs, kv_dtype)
+        per_block = max(1, m.kv_block_bytes(bs, kv_dtype))  # (a model without attention layers holds no KV)
         want_tokens = a.max_batch_seqs * a.max_model_len
         if a.kv_cache_gb:
             budget = int(a.kv_cache_gb * 2 ** 30)
@@ -296,6 +297,8 @@ class InferenceEngine:
             graphs = rows * (m.cfg.vocab_size * 8 + 8 * m.inter + 16 * m.cfg.hidden_size) * 2
             reserve = (6 * 2 ** 30 + 2 * a.prefill_chunk_tokens * (m.cfg.hidden_size + 2 * m.inter) * 2
                        + graphs + self._decode_ws_bytes())
+            if getattr(m, "has_seq_state", False):  # the per-sequence state tables (allocated after the pool)
+                reserve += (rows + 1) * m.state_row_bytes()
             budget = int(min(free - reserve, total * a.gpu_memory_utilization - torch.cuda.memory_allocated(self.device)))
         else:
             budget = 256 * 2 ** 20
@@ -378,6 +381,17 @@ class InferenceEngine:
                            if rows_fn else 64)
         self._tile_rows = getattr(self.model, "prefill_tile_rows", self._tile_rows)
         self._streams: Dict[str, "_Request"] = {}  # open token streams (stream_step), by caller id
+        # models with per-sequence state (recurrences, convolution tails): one table row per state
+        # row of the engine, plus a scratch row that parked and finished rows of a decode bucket
+        # write to (as their KV goes to scratch block 0)
+        self.seq_state = None
+        if getattr(self.model, "has_seq_state", False):
+            self.seq_state = self.model.alloc_state(cap + 1, dev)
+            self._row_ids = torch.arange(cap + 1, dtype=torch.int32, device=dev)
+            self._scratch_row = cap
+
+    def _state_tables(self) -> List[torch.Tensor]:
+        return self.model.state_tensors(self.seq_state) if self.seq_state is not None else []
 
     def _phys(self, blocks: List[int]) -> List[int]:
         return [b + 1 for b in blocks]  # manager ids are shifted past scratch block 0
@@ -468,6 +482,7 @@ class InferenceEngine:
                 if req is None:
                     req = _Request(_Seq(0, [], 0, 0.0, None))
                     req.row, req.pending = self.slots.index(None), True
+                    req.seq.row = req.row
                     self.slots[req.row] = self._streams[sid] = req
                 seq = req.seq
                 a = len(seq.prompt_ids)
@@ -798,13 +813,15 @@ class InferenceEngine:
         admitted = []
         while self._waiting and free and len(admitted) < budget:
             req = self._waiting[0]
-            a = self.blocks.allocate(req.seq.prompt_ids, req.seq.max_new, self.args.prefix_caching)
+            # (a cached prefix holds K / V only: a model with recurrent state must run every token)
+            a = self.blocks.allocate(req.seq.prompt_ids, req.seq.max_new,
+                                     self.args.prefix_caching and self.seq_state is None)
             if not a.ok:
                 break
             self._waiting.popleft()
             req.seq.blocks, req.seq.cached = list(a.blocks), a.num_cached_tokens
             req.seq.done_pos = a.num_cached_tokens
-            req.row = free.pop(0)
+            req.row = req.seq.row = free.pop(0)
             req.pending = True
             self.slots[req.row] = req
             admitted.append(req)
@@ -959,11 +976,11 @@ class InferenceEngine:
             return
         src = self._h2d(torch.tensor(movers, dtype=torch.long))
         dst = self._h2d(torch.tensor(free[:len(movers)], dtype=torch.long))
-        for key, t in self.state.items():
+        for t in list(self.state.values()) + self._state_tables():
             t.index_copy_(0, dst, t.index_select(0, src))
         for a, b in zip(movers, free):
             self.slots[b], self.slots[a] = self.slots[a], None
-            self.slots[b].row = b
+            self.slots[b].row = self.slots[b].seq.row = b
         self._park_rows(movers)
 
     def _block_table(self, seqs: List[_Seq], rows: int) -> torch.Tensor:
@@ -1047,7 +1064,13 @@ class InferenceEngine:
                 tiles.append((b - (q_start[i + 1] - t), i, t, min(t + tr, q_start[i + 1])))
         tiles.sort(key=lambda x: -x[0])
         i32 = torch.int32
+        extra = {}
+        if self.seq_state is not None:
+            seg = [i for i, (_, a, b) in enumerate(chunk) for _ in range(b - a)]
+            extra = dict(state=self.seq_state, state_rows=self._h2d(torch.tensor([wave[r].row for r in rows], dtype=i32)),
+                         token_seq=self._h2d(torch.tensor(seg, dtype=i32)))
         meta = AttnMeta(
+            **extra,
             tiles=self._h2d(torch.tensor([x[1:] for x in tiles], dtype=i32).reshape(-1, 3)),
             single=self._h2d(torch.tensor(single, dtype=i32).reshape(-1, 2)) if split else None,
             positions=self._h2d(torch.cat(pos).to(i32)),
@@ -1094,9 +1117,16 @@ class InferenceEngine:
         attn_lens = None
         if self._skip_done_attn:
             attn_lens = torch.where(st["done"] != 0, torch.ones_like(st["seq_lens"]), st["seq_lens"])
+        extra = {}
+        if self.seq_state is not None:
+            # row i continues state row i; parked and finished rows write the scratch row
+            n = pos.shape[0]
+            ids = self._row_ids[:n]
+            extra = dict(state=self.seq_state, token_seq=ids, q_start=self._row_ids[:n + 1],
+                         state_rows=torch.where(st["done"] != 0, torch.full_like(ids, self._scratch_row), ids))
         return AttnMeta(positions=pos, slots=slots.to(torch.int32), block_tables=st["block_tables"],
                         seq_lens=st["seq_lens"], decode=True, workspace=self.decode_ws, cascade=self.cascade,
-                        attn_seq_lens=attn_lens)
+                        attn_seq_lens=attn_lens, **extra)
 
     def decode_step(self, st: Dict[str, torch.Tensor]):
         """One full decode step (forward + guided sampling), graph-capturable."""

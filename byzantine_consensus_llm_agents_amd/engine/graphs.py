@@ -50,6 +50,8 @@ class DecodeGraphs:
         view = self._views(b)
         # capture-time replays must not disturb live rows: snapshot the state
         saved = {k: v.clone() for k, v in e.state.items()}
+        tables = e._state_tables()  # (recurrent state advances with every replay: restored too)
+        saved_tables = [t.clone() for t in tables]
         if self.pool is None:
             self.pool = torch.cuda.graph_pool_handle()
         side = torch.cuda.Stream()
@@ -63,6 +65,8 @@ class DecodeGraphs:
             e.decode_step(view)
         for k, v in e.state.items():
             v.copy_(saved[k])
+        for t, old in zip(tables, saved_tables):
+            t.copy_(old)
         torch.cuda.synchronize()
         self.captures += 1
         return graph

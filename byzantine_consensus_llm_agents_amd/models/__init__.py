@@ -5,6 +5,9 @@ def model_class(family: str):
     if family == "mofidra":
         from .mofidra import MofidraModel
         return MofidraModel
+    if family == "padadra":
+        from .padadra import PadadraModel
+        return PadadraModel
     from .transformer import DecoderModel
     return DecoderModel
 

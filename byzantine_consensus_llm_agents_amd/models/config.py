@@ -206,6 +206,178 @@ class MofidraConfig:
         return n
 
 
+
+@dataclass(frozen=True)
+class SinkAttentionSpec:
+    """Softmax attention with a learned per-head sink in the denominator, an optional sliding
+    window (``window`` keys: the query's own position and the ``window - 1`` before it; 0 = all),
+    an optional short causal convolution over time on q / k / v (``conv`` taps; 0 = none), one
+    RMS norm over the whole q (and k) projection, interleaved-pair rotary on the first
+    ``rot_dims`` features of every head (``rot_scaling`` = (factor, low, high, original): the
+    wavelength-dependent frequency scaling; None = plain) and values that are rotated by their
+    own position over all ``vdim`` features (the head output is turned back by the query's)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    conv: int = 0
+    window: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_scaling: Optional[tuple] = None
+
+    @property
+    def q_width(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def k_width(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def v_width(self) -> int:
+        return self.kv_heads * self.vdim
+
+
+@dataclass(frozen=True)
+class GatedStateSpec:
+    """A recurrent mixer whose state is one ``dim x vdim`` matrix per head with a decay per key
+    channel.  kind "hgrn2": the forget gate also weights the write (``heads`` q heads, no keys).
+    kind "delta": gated delta rule with ``kv_heads`` q / k heads, a short convolution of ``conv``
+    taps on q / k / v, low-rank decay and output-gate projections (``decay_rank`` / ``gate_rank``
+    are taken from the checkpoint's tensor shapes when one is loaded)."""
+    kind: str
+    heads: int
+    dim: int
+    vdim: int
+    kv_heads: int = 0
+    conv: int = 0
+    decay_rank: int = 0
+    gate_rank: int = 0
+
+
+@dataclass(frozen=True)
+class PadadraLayer:
+    type: str                              # "parallel" | "channel_delta"
+    attn: Optional[SinkAttentionSpec]      # parallel: the left mixer
+    state: GatedStateSpec                  # parallel: the right mixer (hgrn2); channel_delta: the mixer
+    mlp: Optional[FeedForwardSpec]
+
+
+@dataclass(frozen=True)
+class PadadraConfig:
+    """Padadra: every layer is ``x <- x + m (mixer(norm1 x) + ff(norm2 x))`` with scalar-weight
+    norms; the mixer is either a windowed sink attention beside an HGRN2 recurrence ("parallel")
+    or a gated delta rule with per-channel decay ("channel_delta").  The embedding adds a hashed
+    bigram row.  Everything is read from the model directory's config.json."""
+    name: str
+    hidden_size: int
+    vocab_size: int
+    layers: tuple
+    rms_eps: float = 1e-6
+    embed_scale: float = 1.0
+    residual_mult: float = 1.0
+    bigram: Optional[tuple] = None         # (buckets, mul_prev, mul_cur)
+    family: str = "padadra"
+    max_position: int = 1 << 20
+    tie_embeddings: bool = False
+
+    @staticmethod
+    def _attn(m: dict) -> SinkAttentionSpec:
+        rot = m.get("rot") or {}
+        sc = rot.get("scaling")
+        spec = SinkAttentionSpec(
+            heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m["vdim"]),
+            scale=float(m["scale"]), conv=int(m.get("conv") or 0), window=int((m.get("mask") or {}).get("size", 0)),
+            rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)),
+            rot_scaling=None if not sc else tuple(float(sc[k]) for k in ("factor", "low", "high", "original")))
+        if spec.heads % spec.kv_heads or spec.rot_dims % 2 or spec.rot_dims > spec.dim or spec.vdim % 2:
+            raise ValueError("Padadra: heads % kv_heads, rot.dims even and <= dim, vdim even")
+        return spec
+
+    @classmethod
+    def from_dict(cls, c: dict, name: str = "padadra") -> "PadadraConfig":
+        layers = []
+        for entry in c["layers"]:
+            m, kind = entry["mixer"], entry["type"]
+            if kind == "parallel":
+                r = m["right"]
+                attn = cls._attn(m["left"])
+                state = GatedStateSpec("hgrn2", int(r["heads"]), int(r["dim"]), int(r["vdim"]))
+            elif kind == "channel_delta":
+                attn = None
+                state = GatedStateSpec("delta", int(m["heads"]), int(m["dim"]), int(m["vdim"]),
+                                       kv_heads=int(m.get("kv_heads", m["heads"])), conv=int(m.get("conv") or 0),
+                                       decay_rank=int(m.get("decay_rank", 0)), gate_rank=int(m.get("gate_rank", 0)))
+                if state.heads % state.kv_heads:
+                    raise ValueError("Padadra: heads must be a multiple of kv_heads")
+            else:
+                raise ValueError(f"Padadra: unknown layer type {kind!r}")
+            f = entry.get("mlp")
+            if f is not None and f["kind"] != "dense":
+                raise ValueError(f"Padadra: unknown feed-forward kind {f['kind']!r}")
+            layers.append(PadadraLayer(kind, attn, state, FeedForwardSpec("dense", int(f["ff"])) if f else None))
+        emb = c.get("embedding") or {}
+        bg = emb.get("bigram")
+        return cls(name=name, hidden_size=int(c["width"]), vocab_size=int(c["vocab"]), layers=tuple(layers),
+                   rms_eps=float(c["norm"]["eps"]), embed_scale=float(emb.get("scale", 1.0)),
+                   residual_mult=float(c.get("residual_mult", 1.0)),
+                   bigram=(int(bg["buckets"]), int(bg["mul_prev"]), int(bg["mul_cur"])) if bg else None)
+
+    def to_dict(self) -> dict:
+        """The config.json form (inverse of `from_dict`)."""
+        out = []
+        for l in self.layers:
+            s = l.state
+            if l.type == "parallel":
+                a = l.attn
+                left = {"heads": a.heads, "kv_heads": a.kv_heads, "dim": a.dim, "vdim": a.vdim, "scale": a.scale}
+                if a.conv:
+                    left["conv"] = a.conv
+                if a.window:
+                    left["mask"] = {"size": a.window}
+                if a.rot_dims:
+                    left["rot"] = {"dims": a.rot_dims, "base": a.rot_base}
+                    if a.rot_scaling:
+                        left["rot"]["scaling"] = dict(zip(("factor", "low", "high", "original"), a.rot_scaling))
+                else:
+                    left["rot"] = {"dims": 0, "base": a.rot_base}
+                mixer = {"left": left, "right": {"heads": s.heads, "dim": s.dim, "vdim": s.vdim}}
+            else:
+                mixer = {"heads": s.heads, "kv_heads": s.kv_heads, "dim": s.dim, "vdim": s.vdim}
+                if s.conv:
+                    mixer["conv"] = s.conv
+                if s.decay_rank:
+                    mixer["decay_rank"] = s.decay_rank
+                if s.gate_rank:
+                    mixer["gate_rank"] = s.gate_rank
+            out.append({"type": l.type, "mixer": mixer, "mlp": {"kind": "dense", "ff": l.mlp.ff} if l.mlp else None})
+        emb = {"scale": self.embed_scale}
+        if self.bigram:
+            emb["bigram"] = dict(zip(("buckets", "mul_prev", "mul_cur"), self.bigram))
+        return {"architecture": "Padadra", "width": self.hidden_size, "vocab": self.vocab_size, "embedding": emb,
+                "norm": {"eps": self.rms_eps}, "residual_mult": self.residual_mult, "layers": out}
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def num_params(self) -> int:
+        W, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size
+        for l in self.layers:
+            s = l.state
+            if l.attn is not None:
+                a = l.attn
+                n += W * (a.q_width + a.k_width + a.v_width) + W * a.heads * a.vdim
+                n += W * (2 * s.heads * s.dim + s.heads * s.vdim) + W * s.heads * s.vdim
+            else:
+                n += W * (2 * s.kv_heads * s.dim + 2 * s.heads * s.vdim)
+            if l.mlp is not None:
+                n += 2 * W * l.mlp.ff
+        return n
+
+
 PRESETS = {
     "Qwen/Qwen3-8B": ModelConfig("Qwen/Qwen3-8B", "qwen3", 4096, 36, 32, 8, 128, 12288, 151936,
                                  qk_norm=True, max_position=40960),
@@ -241,6 +413,8 @@ def from_hf_config(path: str, name: Optional[str] = None):
         c = json.load(fh)
     if str(c.get("architecture", "")).lower() == "mofidra":
         return MofidraConfig.from_dict(c, name or path)
+    if str(c.get("architecture", "")).lower() == "padadra":
+        return PadadraConfig.from_dict(c, name or path)
     arch = (c.get("model_type") or "").lower()
     family = "qwen3" if arch == "qwen3" else ("qwen2" if arch == "qwen2" else "mistral")
     heads = c["num_attention_heads"]

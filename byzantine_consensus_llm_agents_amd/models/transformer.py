@@ -48,6 +48,12 @@ class AttnMeta:
     # packed steps of models with `split_single_rows`: [n, 2] int32 {token row, sequence} of the
     # one-token segments (a decoded token beside prompt portions); `tiles` then hold the others
     single: Optional[torch.Tensor] = None
+    # models with per-sequence state besides the KV cache (`has_seq_state`): the model's state
+    # tables (its `alloc_state`), every segment's row in them [B] int32 and the segment of every
+    # packed row [T] int32; `q_start` is then given for decode steps too
+    state: Optional[dict] = None
+    state_rows: Optional[torch.Tensor] = None
+    token_seq: Optional[torch.Tensor] = None
 
 
 class TPGroup:

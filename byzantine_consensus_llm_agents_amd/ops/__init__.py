@@ -23,14 +23,14 @@ def _torch_ops() -> SimpleNamespace:
                 tile_rows=64):
         return _ref.paged_attention(q, k_cache, v_cache, layer, block_tables, q_start, seq_lens, scale)
 
-    def multimap_attention(q, k_cache, v_cache, meta, scale, maps, lam, head_eps, out_scale, vdim):
+    def multimap_attention(q, k_cache, v_cache, meta, scale, maps, lam, head_eps, out_scale, vdim, window=0, sink=None):
         # tiles / single-row lists only tell the HIP kernels how to walk the batch
         q_start = meta.q_start
         if q_start is None:  # decode: one row per sequence
             q_start = torch.arange(q.shape[0] + 1, dtype=torch.int32, device=q.device)
         lens = meta.seq_lens if meta.attn_seq_lens is None else meta.attn_seq_lens
         return _ref.multimap_attention(q, k_cache, v_cache, meta.block_tables, q_start, lens, scale, maps,
-                                       lam, head_eps, out_scale, vdim)
+                                       lam, head_eps, out_scale, vdim, window, sink)
 
     return SimpleNamespace(
         name="torch",
@@ -42,6 +42,16 @@ def _torch_ops() -> SimpleNamespace:
         act_fn=_ref.act_fn,
         moe_route=_ref.moe_route,
         moe_experts=_ref.moe_experts,
+        embed_hashed_bigram_norm=_ref.embed_hashed_bigram_norm,
+        rmsnorm_scalar=_ref.rmsnorm_scalar,
+        residual_mix_norm=_ref.residual_mix_norm,
+        short_conv=_ref.short_conv,
+        rope_pairs_kv_write=_ref.rope_pairs_kv_write,
+        rotate_pairs=_ref.rotate_pairs,
+        hgrn2_prepare=_ref.hgrn2_prepare,
+        delta_prepare=_ref.delta_prepare,
+        gated_state_scan=_ref.gated_state_scan,
+        head_norm_gate=_ref.head_norm_gate,
         linear=torch.nn.functional.linear,
         rmsnorm=_ref.rmsnorm,
         add_rmsnorm=_ref.add_rmsnorm,

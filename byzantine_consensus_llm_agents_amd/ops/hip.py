@@ -102,7 +102,26 @@ def load_library(path: str = None) -> ctypes.CDLL:
         "bcg_multimap_split_keys": [],
         "bcg_multimap_attention": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                    c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                   c_float, c_float, c_float, c_float, c_int, c_int, c_void_p],
+                                   c_float, c_float, c_float, c_float, c_int, c_int, c_int, c_void_p, c_void_p],
+        "bcg_embed_hashed_bigram": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float,
+                                    c_void_p, c_int, c_int, c_int, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p,
+                                    c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_residual_mix_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float,
+                                  c_float, c_float, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "bcg_short_conv": [c_void_p, c_int64, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                           c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_rope_pairs_kv_write": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int,
+                                    c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_int, c_void_p],
+        "bcg_rotate_pairs": [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_hgrn2_prepare": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                              c_int, c_int, c_void_p],
+        "bcg_delta_prepare": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                              c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_gated_state_scan": [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_head_norm_gate": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int,
+                               c_void_p],
         "bcg_moe_tile_rows": [],
         "bcg_moe_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                           c_int, c_int, c_void_p],
@@ -572,7 +591,9 @@ def hip_ops() -> SimpleNamespace:
         return residual.add_(linear_fp8(xq, xs, wq, ws))
 
     from .seqmix import seqmix_ops
+    from .seqstate import seqstate_ops
     extra = seqmix_ops(lib, linear)
+    extra.update(seqstate_ops(lib))
 
     return SimpleNamespace(name="hip", **extra, rmsnorm_fp8=rmsnorm_fp8, embed_rmsnorm_fp8=embed_rmsnorm_fp8,
                            linear_fp8_residual=linear_fp8_residual, linear=linear, linear_silu=linear_silu, linear_residual=linear_residual,

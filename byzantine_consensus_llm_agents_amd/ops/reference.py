@@ -405,11 +405,13 @@ def rope_multi_kv_write(qkv, positions, slots, n_q: int, n_kv: int, maps: int, d
 
 
 def multimap_attention(q, k_cache, v_cache, block_tables, q_start, seq_lens, scale: float, maps: int,
-                       lam: float, head_eps: float, out_scale: float, vdim: int):
+                       lam: float, head_eps: float, out_scale: float, vdim: int, window: int = 0, sink=None):
     """Causal GQA attention with ``maps`` softmax maps per head over shared values:
     ``o = a_0 - lam * a_1`` (maps = 2; maps = 1: ``a_0``), then per head
     ``o / sqrt(mean(o^2) + head_eps) * out_scale`` (``head_eps < 0``: only the scale).
-    Sequence b's query rows ``q_start[b]:q_start[b+1]`` are its last positions.  Returns
+    Sequence b's query rows ``q_start[b]:q_start[b+1]`` are its last positions.  ``window`` > 0:
+    position i sees only j with i - j < window.  ``sink`` fp32 [n_q]: the softmax denominator of
+    head h also holds ``exp(sink[h])`` (no key, no value, not scaled).  Returns
     ``[T, n_q * vdim]``; fp32 math."""
     T, n_q, qd = q.shape
     dim = qd // maps
@@ -429,11 +431,19 @@ def multimap_attention(q, k_cache, v_cache, block_tables, q_start, seq_lens, sca
         k, v = k.repeat_interleave(group, 0), v.repeat_interleave(group, 0)
         qb = q[s:e].float().permute(1, 0, 2)
         qpos = torch.arange(ctx - (e - s), ctx, device=q.device)[:, None]
-        hidden = torch.arange(ctx, device=q.device)[None, :] > qpos
+        kpos = torch.arange(ctx, device=q.device)[None, :]
+        hidden = kpos > qpos
+        if window > 0:
+            hidden = hidden | (kpos < qpos - window + 1)
         o = None
         for m in range(maps):
             sc = torch.matmul(qb[..., m * dim:(m + 1) * dim], k[..., m * dim:(m + 1) * dim].transpose(1, 2)) * scale
-            a = torch.matmul(torch.softmax(sc.masked_fill(hidden, float("-inf")), -1), v)
+            sc = sc.masked_fill(hidden, float("-inf"))
+            if sink is not None:
+                col = sink.float()[:, None, None].expand(n_q, e - s, 1)
+                a = torch.matmul(torch.softmax(torch.cat([sc, col], -1), -1)[..., :-1], v)
+            else:
+                a = torch.matmul(torch.softmax(sc, -1), v)
             o = a if m == 0 else o - lam * a
         if head_eps >= 0:
             o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + head_eps)
@@ -442,12 +452,14 @@ def multimap_attention(q, k_cache, v_cache, block_tables, q_start, seq_lens, sca
 
 
 def act_fn(x: torch.Tensor, kind: str) -> torch.Tensor:
-    """"gelu_tanh": 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))); "relu2": max(z, 0)^2."""
+    """"gelu_tanh": 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))); "relu2": max(z, 0)^2; "silu": z sigmoid(z)."""
     z = x.float()
     if kind == "gelu_tanh":
         y = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
     elif kind == "relu2":
         y = torch.relu(z).pow(2)
+    elif kind == "silu":
+        y = z * torch.sigmoid(z)
     else:
         raise ValueError(f"unknown activation {kind!r}")
     return y.to(x.dtype)
@@ -480,3 +492,235 @@ def moe_experts(h, up, down, idx, weights, kind: str = "relu2"):
         y = torch.nn.functional.linear(act_fn(torch.nn.functional.linear(x, up[e]), kind), down[e])
         out.index_add_(0, rows, y.float() * weights[rows, slot][:, None])
     return out
+
+
+# ------------------------------------------------------------------ per-sequence state: hashed bigram, short convolutions,
+# pair rotary with value rotation, gated-state recurrences (models/padadra.py)
+#
+# A packed step holds B segments; segment b is rows ``q_start[b]:q_start[b+1]`` (consecutive
+# positions of one sequence), ``token_seq[t]`` is the segment of row t and ``state_rows[b]`` the
+# row of the per-sequence state tables that the segment continues.  A segment that starts at
+# position 0 starts from empty state whatever the table holds, so a state row needs no reset
+# when it is handed to a new sequence.
+
+def embed_hashed_bigram(tokens, meta, prev, table, scale: float, bigram, hash_mul):
+    """fp32 stream ``scale * E[token] + bigram[row]``; row = (previous token * mul_prev + token *
+    mul_cur) mod buckets, or the table's last row at position 0 (``bigram`` None: no bigram term).
+    ``prev`` int32 [rows]: the last token of every state row; read for a segment's first token,
+    then set to the segment's last token."""
+    x = table.index_select(0, tokens.long()).float() * scale
+    if bigram is None:
+        return x
+    T = tokens.numel()
+    first, last = meta.q_start[:-1].long(), meta.q_start[1:].long() - 1
+    before = torch.zeros(T, dtype=torch.int64, device=tokens.device)
+    before[1:] = tokens[:-1].long()
+    before[first] = prev[meta.state_rows.long()].long()
+    buckets = bigram.shape[0] - 1
+    row = (before * int(hash_mul[0]) + tokens.long() * int(hash_mul[1])) % buckets
+    row = torch.where(meta.positions.long() == 0, torch.full_like(row, buckets), row)
+    prev[meta.state_rows.long()] = tokens[last].to(prev.dtype)
+    return x + bigram.index_select(0, row).float()
+
+
+def embed_hashed_bigram_norm(tokens, meta, prev, table, scale: float, bigram, hash_mul, eps: float, gains, out_dtype):
+    """(`embed_hashed_bigram` stream, its `rmsnorm_scalar` for ``gains``)."""
+    x = embed_hashed_bigram(tokens, meta, prev, table, scale, bigram, hash_mul)
+    return x, rmsnorm_scalar(x, eps, gains, out_dtype)
+
+
+def rmsnorm_scalar(x, eps: float, gains, out_dtype):
+    """``x / sqrt(mean(x^2) + eps) * g`` for every scalar g of ``gains`` (fp32 math)."""
+    xf = x.float()
+    unit = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return tuple((unit * float(g)).to(out_dtype) for g in gains)
+
+
+def residual_mix_norm(x, normed, normed_scale: float, plain, mult: float, eps: float, gains, out_dtype):
+    """``x += mult * (normed_scale * sum_i rms(a_i) * w_i + sum_j p_j)`` in fp32, in place
+    (``normed``: [(a_i [T, W], w_i fp32 [W])], every a_i RMS-normed over the row; ``plain``:
+    [p_j]); returns `rmsnorm_scalar` of the new x for ``gains``."""
+    total = None
+    for a, w in normed:
+        af = a.float()
+        t = af * torch.rsqrt(af.pow(2).mean(-1, keepdim=True) + eps) * w.float() * normed_scale
+        total = t if total is None else total + t
+    for p in plain:
+        total = p.float() if total is None else total + p.float()
+    if total is not None:
+        x.add_(total * mult)
+    return rmsnorm_scalar(x, eps, gains, out_dtype)
+
+
+def short_conv(y, channels: int, w, meta, state, act=None):
+    """Causal convolution over time on the first ``channels`` columns of ``y`` [T, >= channels]:
+    ``out_t = sum_j w[:, j] u_(t - taps + 1 + j)`` (fp32 sum, rounded once), zeros before position
+    0, then ``act`` (None | "silu").  ``state`` [rows, taps - 1, channels]: the last inputs of
+    every state row; read where a segment reaches before its first row, then updated."""
+    T, taps = y.shape[0], w.shape[1]
+    u = y[:, :channels]
+    seg = meta.token_seq.long()
+    qs = meta.q_start.long()
+    t_idx = torch.arange(T, device=y.device)
+    off = t_idx - qs[seg]                      # row's offset in its segment
+    rows = meta.state_rows.long()
+    pos = meta.positions.long()
+    acc = torch.zeros(T, channels, dtype=torch.float32, device=y.device)
+    for j in range(taps):
+        back = taps - 1 - j
+        in_seg = off >= back
+        val = u[(t_idx - back).clamp(min=0)].float()
+        if taps > 1:
+            old = state[rows[seg], (j + off).clamp(max=taps - 2)].float()
+            val = torch.where(in_seg[:, None], val, torch.where((pos - back >= 0)[:, None], old, torch.zeros_like(old)))
+        acc += w[:, j].float()[None, :] * val
+    if taps > 1:
+        new = torch.zeros(rows.numel(), taps - 1, channels, dtype=torch.float32, device=y.device)
+        n = qs[1:] - qs[:-1]
+        pos0 = pos[qs[:-1]]
+        for i in range(taps - 1):
+            b = taps - 1 - i
+            fresh = u[(qs[1:] - b).clamp(min=0)].float()
+            old = state[rows, (i + n).clamp(max=taps - 2)].float() * (pos0 > 0)[:, None]
+            new[:, i] = torch.where((n >= b)[:, None], fresh, old)
+        state[rows] = new.to(state.dtype)
+    if act == "silu":
+        acc = acc * torch.sigmoid(acc)
+    elif act is not None:
+        raise ValueError(f"unknown activation {act!r}")
+    return acc.to(y.dtype)
+
+
+def scaled_inv_freq(dims: int, base: float, scaling=None, device=None) -> torch.Tensor:
+    """fp32 ``base^(-2i/dims)``; with ``scaling`` = (factor, low, high, original) a frequency whose
+    wavelength l = 2 pi / f is above original / low is divided by factor, one below original /
+    high is kept, and between them s = (original / l - low) / (high - low) blends
+    ``(1 - s) f / factor + s f``."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / max(dims, 1))
+    if scaling is not None:
+        factor, low, high, orig = (float(v) for v in scaling)
+        wl = 2.0 * math.pi / f
+        s = ((orig / wl - low) / (high - low)).clamp(0.0, 1.0)
+        mid = (1.0 - s) * f / factor + s * f
+        f = torch.where(wl < orig / high, f, torch.where(wl > orig / low, f / factor, mid))
+    return f.float().to(device)
+
+
+def _turn_pairs(x, ang):
+    """x [..., 2n]: the pair (2i, 2i + 1) turned by ang[..., i]."""
+    a, b = x[..., 0::2], x[..., 1::2]
+    c, s = ang.cos(), ang.sin()
+    return torch.stack([a * c - b * s, b * c + a * s], dim=-1).flatten(-2)
+
+
+def rope_pairs_kv_write(qkv, positions, slots, n_q: int, n_kv: int, dim: int, vdim: int, q_norm, k_norm, eps: float,
+                        inv_freq, v_inv_freq, k_cache, v_cache):
+    """Row ``[q | k | v | ...]``: one RMS norm over the whole q part (weight ``q_norm``
+    [n_q dim]; None = no norm) and one over the whole k part, then every q / k head's features
+    (2i, 2i + 1), i < len(inv_freq), are turned by ``position * inv_freq[i]``; every v head's pairs
+    by ``position * v_inv_freq[i]`` (None: values as they are).  K / V go to the paged cache of
+    `rope_multi_kv_write`; returns q [T, n_q, dim]."""
+    T = qkv.shape[0]
+    qw, kw = n_q * dim, n_kv * dim
+    q, k = qkv[:, :qw].float(), qkv[:, qw:qw + kw].float()
+    v = qkv[:, qw + kw:qw + kw + n_kv * vdim].float().reshape(T, n_kv, vdim)
+    if q_norm is not None:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm.float()
+    if k_norm is not None:
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm.float()
+    q, k = q.reshape(T, n_q, dim), k.reshape(T, n_kv, dim)
+    pos = positions.float()[:, None, None]
+    r = 2 * inv_freq.numel()
+    if r:
+        ang = pos * inv_freq.float()[None, None, :]
+        q = torch.cat([_turn_pairs(q[..., :r], ang), q[..., r:]], -1)
+        k = torch.cat([_turn_pairs(k[..., :r], ang), k[..., r:]], -1)
+    if v_inv_freq is not None:
+        v = _turn_pairs(v, pos * v_inv_freq.float()[None, None, :])
+    bs = k_cache.shape[2]
+    blk, off = (slots // bs).long(), (slots % bs).long()
+    k_cache[blk, :, off] = k.to(k_cache.dtype)
+    v_cache[blk, :, :, off] = v.to(v_cache.dtype)
+    return q.to(qkv.dtype)
+
+
+def rotate_pairs(x, positions, inv_freq, sign: float, heads: int):
+    """x [T, heads * 2n]: every head's pair (2i, 2i + 1) turned by ``sign * position * inv_freq[i]``."""
+    T = x.shape[0]
+    xf = x.float().reshape(T, heads, -1)
+    ang = sign * positions.float()[:, None, None] * inv_freq.float()[None, None, :]
+    return _turn_pairs(xf, ang).reshape(T, -1).to(x.dtype)
+
+
+def hgrn2_prepare(y, off_q: int, off_f: int, heads: int, dim: int, f_bias, lower):
+    """From a fused projection row: ``q = silu(y_q)``, forget gate ``f = l + (1 - l) sigmoid(y_f +
+    bias)``; returns fp32 (q, 1 - f, f), each [T, heads, dim]: the read, write and decay vectors of
+    `gated_state_scan`."""
+    T, n = y.shape[0], heads * dim
+    q = y[:, off_q:off_q + n].float()
+    q = q * torch.sigmoid(q)
+    low = lower.float()
+    f = low + (1.0 - low) * torch.sigmoid(y[:, off_f:off_f + n].float() + f_bias.float())
+    return q.reshape(T, heads, dim), (1.0 - f).reshape(T, heads, dim), f.reshape(T, heads, dim)
+
+
+def delta_prepare(c, y, off_beta: int, a, a_log, dt_bias, heads: int, kv_heads: int, dim: int):
+    """``c`` [T, >= 2 kv_heads dim]: q | k after convolution and activation; every q / k head
+    becomes a unit vector ``x / sqrt(sum x^2 + 1e-6)`` (q also times dim^-1/2); ``beta = sigmoid(y
+    [:, off_beta + h])``; decay ``g = exp(-exp(a_log[h]) softplus(a + dt_bias))`` per head and key
+    channel (``a`` [T, heads dim]).  Returns fp32 (q [T, kv_heads, dim], k, g [T, heads, dim], beta [T, heads])."""
+    T, n = c.shape[0], kv_heads * dim
+    q = c[:, :n].float().reshape(T, kv_heads, dim)
+    k = c[:, n:2 * n].float().reshape(T, kv_heads, dim)
+    q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * dim ** -0.5
+    k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+    beta = torch.sigmoid(y[:, off_beta:off_beta + heads].float())
+    sp = torch.nn.functional.softplus(a.float() + dt_bias.float()).reshape(T, heads, dim)
+    g = torch.exp(-torch.exp(a_log.float())[None, :, None] * sp)
+    return q, k, g, beta
+
+
+def gated_state_scan(q, k, g, v, beta, meta, state, delta: bool):
+    """Per head a ``dim x vdim`` fp32 state S with a decay per key channel, token after token:
+
+        S <- diag(g_t) S;   u = v_t                      (delta False)
+                            u = beta_t (v_t - S^T k_t)   (delta True)
+        S <- S + k_t u^T;   o_t = S^T q_t
+
+    q / k [T, Gq, dim] fp32 (head h reads q / k head h // (H / Gq)), g [T, H, dim] fp32, v [T, H
+    vdim], beta [T, H] fp32 or None; ``state`` [rows, H, dim, vdim] fp32 is read (unless the
+    segment starts at position 0) and left at the segment's last token.  Returns fp32 o [T, H, vdim]."""
+    T, H, dim = g.shape
+    vdim = state.shape[3]
+    per = H // q.shape[1]
+    vf = v.float().reshape(T, H, vdim)
+    qh, kh = q.repeat_interleave(per, 1), k.repeat_interleave(per, 1)
+    out = torch.zeros(T, H, vdim, dtype=torch.float32, device=g.device)
+    qs = meta.q_start.tolist()
+    rows = meta.state_rows.tolist()
+    pos = meta.positions.tolist()
+    for b in range(len(rows)):
+        s, e = qs[b], qs[b + 1]
+        if e <= s:
+            continue
+        S = state[rows[b]].clone() if pos[s] > 0 else torch.zeros_like(state[rows[b]])
+        for t in range(s, e):
+            S = S * g[t][:, :, None]
+            u = vf[t]
+            if delta:
+                u = beta[t][:, None] * (u - torch.einsum("hde,hd->he", S, kh[t]))
+            S = S + kh[t][:, :, None] * u[:, None, :]
+            out[t] = torch.einsum("hde,hd->he", S, qh[t])
+        state[rows[b]] = S
+    return out
+
+
+def head_norm_gate(o, w, eps: float, gate, out_dtype):
+    """o fp32 [T, H, vdim]: every head divided by its root mean square, times ``w`` [vdim], times
+    ``sigmoid(gate)`` (gate [T, H vdim] logits or None); returns [T, H vdim] in ``out_dtype``."""
+    T, H, vdim = o.shape
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    if gate is not None:
+        y = y * torch.sigmoid(gate.float().reshape(T, H, vdim))
+    return y.reshape(T, H * vdim).to(out_dtype)

@@ -84,7 +84,7 @@ def seqmix_ops(lib, linear):
         _req(x.dim() == 2 and x.stride(1) == 1, "act_fn: [rows, n] with unit column stride")
         rows, n = x.shape
         out = torch.empty(rows, n, dtype=x.dtype, device=x.device)
-        code = {"gelu_tanh": 0, "relu2": 1}[kind]
+        code = {"gelu_tanh": 0, "relu2": 1, "silu": 2}[kind]
         _check(lib.bcg_act_fn(_p(x), _p(out), rows, n, x.stride(0), code, _act(x), _stream()), "act_fn")
         return out
 
@@ -137,9 +137,10 @@ def seqmix_ops(lib, linear):
         """Query rows per prefill tile (the tile table the engine builds) for these head sizes."""
         return 64  # four waves x 16 rows
 
-    def multimap_attention(q, k_cache, v_cache, meta, scale, maps, lam, head_eps, out_scale, vdim):
+    def multimap_attention(q, k_cache, v_cache, meta, scale, maps, lam, head_eps, out_scale, vdim, window=0, sink=None):
         """Prefill tiles (``meta.tiles``) on the MFMA kernel, one-token rows (``meta.single``, or
-        every row of a decode step) on the split-KV kernel."""
+        every row of a decode step) on the split-KV kernel.  ``window`` / ``sink`` (one-map heads):
+        sliding window in keys, fp32 [H] sink logits of the softmax denominator."""
         T, H, qd = q.shape
         _req(q.is_contiguous() and qd % maps == 0, "q [T, H, maps dim] contiguous")
         dim = qd // maps
@@ -154,10 +155,16 @@ def seqmix_ops(lib, linear):
         f32 = _act(q)
         tile_rows = meta.tile_rows if not meta.decode else 64
         _req(tile_rows == 64, "prefill tiles: 64 query rows")
-        common = (H, G, maps, dim, vdim, BS, NB, scale, lam, head_eps, out_scale, tile_rows, f32, _stream())
+        window = int(window or 0)
+        _req(window >= 0 and (maps == 1 or (window == 0 and sink is None)), "window / sink: one-map heads")
+        if sink is not None:
+            _req(sink.dtype == torch.float32 and sink.numel() == H and sink.is_contiguous(), "sink fp32 [H]")
+        common = (H, G, maps, dim, vdim, BS, NB, scale, lam, head_eps, out_scale, tile_rows, f32, window, _p(sink), _stream())
 
         def decode(work, n_items):
             n_splits = max(1, (bt.shape[1] * BS + split_keys - 1) // split_keys)
+            if window:  # splits are counted from the window's first: it touches this many at most
+                n_splits = min(n_splits, (window + split_keys - 1) // split_keys + 1)
             ws = torch.empty(n_items * H * n_splits * (2 * maps + maps * vdim), dtype=torch.float32, device=q.device)
             _check(lib.bcg_multimap_attention(1, _p(q), _p(k_cache), _p(v_cache), _p(bt), bt.shape[1], None, _p(lens),
                                               _p(work), n_items, _p(out), _p(ws), n_splits, *common), "multimap decode")

@@ -24,6 +24,11 @@
 // one KV head (GQA packing), so the cache is read once per KV head; one wave per 128-key split.
 // The split size is fixed, so a row's result does not depend on what else is in the batch.
 // decode_merge_kernel merges the splits and applies the map combination + head norm.
+//
+// Optional, for one-map heads: a sliding window (a query at position i sees keys j with
+// i - j < window) and a per-head sink, a learned logit that takes part in the softmax denominator
+// only (no key, no value, not scaled).  The key loop starts at the window's first 16-key tile;
+// decode splits are counted from the window's first split.
 #include <algorithm>
 
 #include "seqmix_common.h"
@@ -31,6 +36,8 @@
 namespace {
 
 constexpr int SPLIT_KEYS = 128;
+constexpr float MAX_FLOOR = -1.0e30f;   // running maxima start finite: a tile may be hidden as a whole
+constexpr float LOG2E = 1.4426950408889634f;
 
 struct AttnArgs {
   const void* q;            // [T, H, maps dim]
@@ -45,12 +52,15 @@ struct AttnArgs {
   int max_blocks, H, G, maps, dim, vdim, BS, num_blocks, n_splits;
   float scale, lam, head_eps, out_scale;
   int vec_k, vec_v;         // rows of K / V^T are aligned for 4-element vector loads
+  int window;               // > 0: keys below position - window + 1 are hidden
+  const float* sink;        // [H] or null
   int swz;                  // fragment-major slabs (see the top of the file)
 };
 
 // The key loop shared by both kernels: keys [k_begin, k_last] of one sequence for the 16 query
 // columns of a wave (column = a query row of one head, or a query head of one token).
 //   limit      per lane: the last key its column may see;  limit_min: the smallest over the wave
+//   lo         per lane: the first key its column may see;  lo_max: the largest over the wave
 //   KT         16-key tiles per iteration (one softmax update and one rescale per iteration)
 //   PF         this iteration's V^T fragments are loaded before its QK^T products and the next
 //              iteration's K fragments right after them (loads fly under the MFMAs and the softmax)
@@ -60,7 +70,7 @@ struct AttnArgs {
 // log2 domain (scale * log2 e folded into one multiply, v_exp_f32 directly).
 template <typename T, int KC, int VT, int KT, bool PF, bool FULL, bool EXACT>
 __device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const typename Elem<T>::frag (&qf)[2][KC],
-                                             int limit, int limit_min, int k_begin, int k_last,
+                                             int limit, int limit_min, int lo, int lo_max, int k_begin, int k_last,
                                              const int* __restrict__ table, f32x4 (&acc)[2][VT], float (&mx)[2],
                                              float (&den)[2]) {
   typedef typename Elem<T>::frag F;
@@ -159,7 +169,7 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const ty
     // softmax and the second product
     if (PF && key0 + 16 * KT <= k_last) load_k(k_cur, kf);
     // ---- online softmax per query column; lane holds keys key0 + 16 u + 4 grp + i ----
-    const bool masked = key0 + 16 * KT - 1 > limit_min;     // (wave-uniform) some key of the iteration is hidden
+    const bool masked = key0 + 16 * KT - 1 > limit_min || key0 < lo_max;   // (wave-uniform) some key of the iteration is hidden
     F pf[KT][2];
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
@@ -174,12 +184,12 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const ty
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           v[u][i] = s[u][m][i] * sc;
-          if (masked && key0 + 16 * u + 4 * grp + i > limit) v[u][i] = -INFINITY;
+          if (masked && (key0 + 16 * u + 4 * grp + i > limit || key0 + 16 * u + 4 * grp + i < lo)) v[u][i] = -INFINITY;
           bm = fmaxf(bm, v[u][i]);
         }
       bm = fmaxf(bm, __shfl_xor(bm, 16, WAVE));
       bm = fmaxf(bm, __shfl_xor(bm, 32, WAVE));
-      const float m_new = fmaxf(mx[m], bm);                 // finite: the range's first key is visible
+      const float m_new = fmaxf(mx[m], bm);                 // finite: the running maximum starts finite
       float ps = 0.f;
 #pragma unroll
       for (int u = 0; u < KT; ++u)
@@ -247,8 +257,14 @@ __global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
   for (int m = 0; m < 2; ++m)
 #pragma unroll
     for (int t = 0; t < VT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float mx[2] = {-INFINITY, -INFINITY}, den[2] = {0.f, 0.f};
-  attend_range<T, KC, VT, KT, PF, FULL, EXACT>(a, g, qf, pos, pos_min, 0, pos_max,
+  float mx[2] = {MAX_FLOOR, MAX_FLOOR}, den[2] = {0.f, 0.f};
+  if (a.sink != nullptr) {   // the sink starts the softmax: weight 1 at its own logit
+    mx[0] = a.sink[h] * LOG2E;
+    den[0] = 1.0f;
+  }
+  const int lo = a.window > 0 ? pos - a.window + 1 : 0, lo_max = a.window > 0 ? pos_max - a.window + 1 : 0;
+  const int k_begin = a.window > 0 ? (max(0, pos_min - a.window + 1) & ~15) : 0;
+  attend_range<T, KC, VT, KT, PF, FULL, EXACT>(a, g, qf, pos, pos_min, lo, lo_max, k_begin, pos_max,
                                         a.block_tables + static_cast<size_t>(seq) * a.max_blocks, acc, mx, den);
   // ---- combine the maps, unit norm over the head's value features, store ----
   const float i0 = 1.0f / den[0], i1 = a.maps > 1 ? a.lam / den[1] : 0.f;
@@ -294,7 +310,10 @@ __global__ __launch_bounds__(64, OCC) void decode_mfma_kernel(AttnArgs a) {
   const int split = blockIdx.y, item = blockIdx.z;
   const int row = a.work ? a.work[2 * item] : item, seq = a.work ? a.work[2 * item + 1] : item;
   const int ctx = a.seq_lens[seq];
-  const int k_begin = split * SPLIT_KEYS, k_end = min(ctx, k_begin + SPLIT_KEYS);
+  const int lo = a.window > 0 ? max(0, ctx - a.window) : 0;          // first visible key
+  const int split_abs = lo / SPLIT_KEYS + split;                      // splits count from the window's first
+  const int k_end = min(ctx, (split_abs + 1) * SPLIT_KEYS);
+  const int k_begin = max(split_abs * SPLIT_KEYS, lo & ~15);
   if (k_begin >= k_end) return;
   const bool col_ok = 16 * cg + col < per;
   const int h = g * per + min(16 * cg + col, per - 1);
@@ -315,8 +334,8 @@ __global__ __launch_bounds__(64, OCC) void decode_mfma_kernel(AttnArgs a) {
   for (int m = 0; m < 2; ++m)
 #pragma unroll
     for (int t = 0; t < VT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float mx[2] = {-INFINITY, -INFINITY}, den[2] = {0.f, 0.f};
-  attend_range<T, KC, VT, KT, PF, FULL, EXACT>(a, g, qf, k_end - 1, k_end - 1, k_begin, k_end - 1,
+  float mx[2] = {MAX_FLOOR, MAX_FLOOR}, den[2] = {0.f, 0.f};
+  attend_range<T, KC, VT, KT, PF, FULL, EXACT>(a, g, qf, k_end - 1, k_end - 1, lo, lo, k_begin, k_end - 1,
                                         a.block_tables + static_cast<size_t>(seq) * a.max_blocks, acc, mx, den);
   if (!col_ok) return;
   float* w = a.ws + ((static_cast<size_t>(item) * a.H + h) * a.n_splits + split) * (2 * a.maps + a.maps * a.vdim);
@@ -345,16 +364,18 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(AttnArgs a) {
   const int lane = threadIdx.x, h = blockIdx.x, item = blockIdx.y;
   const int row = a.work ? a.work[2 * item] : item, seq = a.work ? a.work[2 * item + 1] : item;
   const int ctx = a.seq_lens[seq];
-  const int n = min(a.n_splits, (ctx + SPLIT_KEYS - 1) / SPLIT_KEYS);
+  const int s_first = a.window > 0 ? max(0, ctx - a.window) / SPLIT_KEYS : 0;
+  const int n = min(a.n_splits, (ctx + SPLIT_KEYS - 1) / SPLIT_KEYS - s_first);
+  const float sink = a.sink != nullptr ? a.sink[h] * LOG2E : MAX_FLOOR;
   const int stride = 2 * a.maps + a.maps * a.vdim;
   const float* w = a.ws + (static_cast<size_t>(item) * a.H + h) * a.n_splits * stride;
   float o[VPL];
 #pragma unroll
   for (int j = 0; j < VPL; ++j) o[j] = 0.f;
   for (int m = 0; m < a.maps; ++m) {
-    float mx = -INFINITY;
+    float mx = m == 0 ? sink : MAX_FLOOR;
     for (int s = 0; s < n; ++s) mx = fmaxf(mx, w[s * stride + m]);
-    float den = 0.f, num[VPL];
+    float den = (m == 0 && a.sink != nullptr) ? exp2f(sink - mx) : 0.f, num[VPL];
 #pragma unroll
     for (int j = 0; j < VPL; ++j) num[j] = 0.f;
     for (int s = 0; s < n; ++s) {
@@ -455,8 +476,9 @@ BCG_API int bcg_multimap_attention(int mode, const void* q, const void* k_cache,
                                    const void* block_tables, int max_blocks, const void* q_start, const void* seq_lens,
                                    const void* work, int n_work, void* out, void* ws, int n_splits, int H, int G, int maps,
                                    int dim, int vdim, int BS, int num_blocks, float scale, float lam, float head_eps,
-                                   float out_scale, int tile_rows, int is_f32, void* stream) {
+                                   float out_scale, int tile_rows, int is_f32, int window, const void* sink, void* stream) {
   if (n_work <= 0) return 0;
+  if ((window > 0 || sink != nullptr) && maps != 1) return -2;
   if (maps < 1 || maps > 2 || dim > 128 || vdim > 256 || BS % 16 || H % G || n_work > 65535 * 16) return -2;
   AttnArgs a;
   a.q = q; a.k_cache = k_cache; a.v_cache = v_cache;
@@ -469,6 +491,7 @@ BCG_API int bcg_multimap_attention(int mode, const void* q, const void* k_cache,
   a.vec_k = ((maps * dim) % 4 == 0) ? 1 : 0;
   a.vec_v = 1;  // BS % 16 == 0: every 4-key group of a V^T row is aligned
   a.swz = a.vec_k;
+  a.window = window; a.sink = static_cast<const float*>(sink);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (mode == 0) return is_f32 ? launch_prefill<float>(a, n_work, tile_rows, s) : launch_prefill<bf16_t>(a, n_work, tile_rows, s);
   if (n_splits < 1 || H > 65535 || n_splits > 65535 || n_work > 65535) return -2;

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(NT) void residual_norm_kernel(float* __restrict__ r
   for (int i = threadIdx.x; i < W; i += NT) o[i] = Elem<T>::st(x[i] * r * (w_offset + w[i]));
 }
 
-// kind 0: gelu (tanh form); 1: relu squared.  in rows have stride `in_stride`, out is dense.
+// kind 0: gelu (tanh form); 1: relu squared; 2: silu.  in rows have stride `in_stride`, out is dense.
 template <typename T>
 __global__ __launch_bounds__(NT) void act_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t rows, int n,
                                                  int64_t in_stride, int kind) {
@@ -84,6 +84,8 @@ __global__ __launch_bounds__(NT) void act_kernel(const T* __restrict__ in, T* __
     float y;
     if (kind == 0) {
       y = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    } else if (kind == 2) {
+      y = z / (1.0f + expf(-z));
     } else {
       const float p = fmaxf(z, 0.f);
       y = p * p;
