@@ -1,0 +1,116 @@
+"""Padadra on the HIP backend against the float64 oracle: packed steps of the engine (prompt
+portions beside single tokens, page and state-row reuse), fp32 (exact mode) and bf16, and greedy
+generation through the scheduler with captured decode graphs."""
+import numpy as np
+import pytest
+import torch
+
+import padadra_cases as C
+import padadra_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", params=[(n, d) for n in C.CASES for d in ("float32", "bfloat16")],
+                ids=lambda p: f"{p[0]}-{p[1]}")
+def case(request, tmp_path_factory):
+    name, dtype = request.param
+    path = str(tmp_path_factory.mktemp(name))
+    cfg = C.CASES[name]
+    sd = O.to_f64(C.checkpoint(cfg, path, seed=len(name)))
+    eng = C.engine(path, backend="hip", dtype=getattr(torch, dtype))
+    assert eng.ops.name == "hip"
+    yield cfg, sd, eng, dtype
+    eng.shutdown()
+
+
+def _close(got, want, dtype):
+    got = got.double().cpu().numpy()
+    if dtype == "float32":
+        np.testing.assert_allclose(got, want, atol=3e-3, rtol=3e-3)
+    else:  # bf16 activations: error relative to the spread of the logits
+        err = np.sqrt(((got - want) ** 2).mean(-1)) / want.std()
+        assert float(err.max()) < 0.08, float(err.max())
+        assert float(np.median(err)) < 0.03
+
+
+def test_whole_prompt_every_position(case):
+    cfg, sd, eng, dtype = case
+    toks = C.tokens(150, cfg["vocab"], 1)
+    got = eng.stream_step([("a", toks, list(range(150)))], end=["a"])
+    _close(got, O.forward(sd, cfg, toks), dtype)
+
+
+def test_portions_then_single_tokens(case):
+    cfg, sd, eng, dtype = case
+    toks = C.tokens(140, cfg["vocab"], 2)
+    want = O.forward(sd, cfg, toks)
+    at = 0
+    for s in [2, 3, 64, 1, 17, 2, 1]:
+        _close(eng.stream_step([("p", toks[at:at + s], list(range(s)))]), want[at:at + s], dtype)
+        at += s
+    got = [eng.stream_step([("p", toks[p:p + 1], [0])], end=["p"] if p == 139 else []) for p in range(at, 140)]
+    _close(torch.cat(got), want[at:140], dtype)
+
+
+def test_first_tokens_one_by_one(case):
+    cfg, sd, eng, dtype = case
+    toks = C.tokens(6, cfg["vocab"], 4)
+    want = O.forward(sd, cfg, toks)
+    for p in range(6):
+        _close(eng.stream_step([("f", toks[p:p + 1], [0])], end=["f"] if p == 5 else []), want[p:p + 1], dtype)
+
+
+def test_mixed_batches_and_reuse(case):
+    cfg, sd, eng, dtype = case
+    lens = [70, 33, 18, 64, 41, 90, 5, 36, 120]
+    reqs = {f"r{i}": C.tokens(n, cfg["vocab"], 10 + i) for i, n in enumerate(lens)}
+    want = {k: O.forward(sd, cfg, t) for k, t in reqs.items()}
+    at = {k: 0 for k in reqs}
+    waiting, live, step = list(reqs), [], 0
+    free_at_start = eng.blocks.num_free_blocks
+    while waiting or live:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        entries, end, expect = [], [], []
+        for j, k in enumerate(live):
+            if (step + j) % 5 == 4 and at[k] > 0:
+                continue
+            take = [1, 2, 16, 7, 1, 19][(step + j) % 6] if at[k] > 0 else [20, 3, 16][j % 3]
+            take = min(take, len(reqs[k]) - at[k])
+            entries.append((k, reqs[k][at[k]:at[k] + take], list(range(take))))
+            expect.append(want[k][at[k]:at[k] + take])
+            at[k] += take
+            if at[k] == len(reqs[k]):
+                end.append(k)
+        if entries:
+            _close(eng.stream_step(entries, end), np.concatenate(expect), dtype)
+        live = [k for k in live if k not in end]
+        step += 1
+    assert eng.blocks.num_free_blocks == free_at_start and not any(eng.slots)
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+def test_greedy_generation(tmp_path, graphs):
+    """Captured decode graphs: replays advance the recurrent state exactly once per step (the
+    capture's warm-up runs are rolled back), finished rows write the scratch state row."""
+    cfg = C.CASES["mixed"]
+    path = str(tmp_path / "m")
+    sd = O.to_f64(C.checkpoint(cfg, path, seed=2))
+    eng = C.engine(path, backend="hip", dtype=torch.float32, rows=4, use_hip_graphs=graphs, precapture_graphs=False)
+    try:
+        prompts = [C.tokens(n, cfg["vocab"], 20 + n) for n in (9, 31, 16, 2, 40, 23)]
+        budget = [6, 12, 19, 5, 3, 10]
+        outs = eng.generate_ids(prompts, max_tokens=budget, temperature=0.0)
+        for p, out, n in zip(prompts, outs, budget):
+            assert len(out) == n
+            seq = list(p)
+            for tok in out:
+                logits = O.forward(sd, cfg, seq)[-1]
+                top2 = np.sort(logits)[-2:]
+                if float(top2[1] - top2[0]) < 0.05 * float(logits.std()):
+                    break  # the sampler reads bf16 rows: a near tie may go either way
+                assert tok == int(logits.argmax())
+                seq.append(tok)
+    finally:
+        eng.shutdown()
