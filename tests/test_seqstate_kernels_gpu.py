@@ -109,7 +109,7 @@ def test_rope_pairs_kv_write_and_rotate_back(ops, dtype, H, G, d, e, rot):
 
 def _attention_inputs(H, G, d, e, lens, q_lens, dtype, seed, loud=None):
     """Paged K / V of sequences of ``lens`` tokens (shuffled pages), queries for their last
-    ``q_lens`` positions; ``loud`` = (sequence, key position): that key lines up with every query."""
+    ``q_lens`` positions; ``loud`` = (sequence, key position): that key lines up with the sequence's last query."""
     g = torch.Generator().manual_seed(seed)
     BS = 16
     nblk = [(n + BS - 1) // BS for n in lens]
@@ -123,7 +123,7 @@ def _attention_inputs(H, G, d, e, lens, q_lens, dtype, seed, loud=None):
         at += nblk[b]
         k, v = torch.randn(n, G, d, generator=g), torch.randn(n, G, e, generator=g)
         if loud is not None and loud[0] == b:
-            k[loud[1]] = 3.0 * q[sum(q_lens[:b]):sum(q_lens[:b + 1])].mean((0, 1))
+            k[loud[1]] = 2.0 * q[sum(q_lens[:b + 1]) - 1, ::H // G]   # lines up with the first head of every group
             v[loud[1]] = 5.0
         for p in range(n):
             kc[tables[b, p // BS], :, p % BS] = k[p]
