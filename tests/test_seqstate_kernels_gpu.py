@@ -123,7 +123,7 @@ def _attention_inputs(H, G, d, e, lens, q_lens, dtype, seed, loud=None):
         at += nblk[b]
         k, v = torch.randn(n, G, d, generator=g), torch.randn(n, G, e, generator=g)
         if loud is not None and loud[0] == b:
-            k[loud[1]] = 2.0 * q[sum(q_lens[:b + 1]) - 1, ::H // G]   # lines up with the first head of every group
+            k[loud[1]] = 4.0 * q[sum(q_lens[:b + 1]) - 1, ::H // G]   # lines up with the first head of every group
             v[loud[1]] = 5.0
         for p in range(n):
             kc[tables[b, p // BS], :, p % BS] = k[p]
@@ -144,7 +144,7 @@ def test_window_and_sink_attention(ops, dtype, H, G, d, e, window):
     lens, q_lens = [300, 139, 64, 17, 210], [130, 1, 64, 1, 2]
     loud = (1, 139 - window) if 0 < window < 139 else (0, 3)        # first key outside row 1's window
     q, kc, vc, tables, qs, sl = _attention_inputs(H, G, d, e, lens, q_lens, dtype, window + H, loud)
-    sink = torch.randn(H, generator=torch.Generator().manual_seed(5)) * 2
+    sink = 3.0 + torch.randn(H, generator=torch.Generator().manual_seed(5)) * 2
     want = ref.multimap_attention(q, kc, vc, tables, qs, sl, d ** -0.5, 1, 0.0, -1.0, 1.0, e, window, sink)
     kd, vd = ops.kv_from_logical(kc.to(DEV), vc.to(DEV))
     tiles, single = [], []
@@ -168,7 +168,7 @@ def test_window_and_sink_attention(ops, dtype, H, G, d, e, window):
     gd = ops.multimap_attention(q[last].contiguous().to(DEV), kd, vd, dmeta, d ** -0.5, 1, 0.0, -1.0, 1.0, e, window, sink.to(DEV))
     torch.testing.assert_close(gd.cpu().float(), want[last].float(), **tol)
     no_sink = ops.multimap_attention(q[last].contiguous().to(DEV), kd, vd, dmeta, d ** -0.5, 1, 0.0, -1.0, 1.0, e, window, None)
-    assert float((no_sink.cpu().float() - want[last].float()).abs().max()) > 0.05   # the sink is not a no-op here
+    assert float((no_sink.cpu().float() - want[last].float())[2:].abs().max()) > 0.1   # the sink is not a no-op here
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
