@@ -1,5 +1,5 @@
-"""Prefill / decode throughput of the Mofidra family beside the Qwen3-style decoder at equal
-layer sizes (random weights, synthetic tokens), and the hot kernels of both against their
+"""Prefill / decode throughput of the Mofidra and Padadra families beside the Qwen3-style decoder
+at equal layer sizes (random weights, synthetic tokens), and the hot kernels against their
 rooflines.  ``bench.py --family-compare`` prints the result as one JSON line.
 
 Equal size: same width, layers, query / KV heads, 128 features per query head (Mofidra: two
@@ -7,8 +7,16 @@ Equal size: same width, layers, query / KV heads, 128 features per query head (M
 matrices, the dense gelu layer two; the MoE variant routes top-2 of 8 experts of ff/4 plus an
 always-on expert of ff/2, i.e. the dense layer's active parameters).
 
+Padadra at equal size: the same width, query / KV heads and feed-forward width; the attention
+mixer has 128 query / key features and 128 value features per head, a 512-key window and 4-tap
+convolutions; the HGRN2 mixer beside it has half as many heads of 64 x 128 state; the gated delta
+rule has the query-head count, half as many q / k heads, 128 x 128 state and 4-tap convolutions;
+one layer in four is a delta layer.  Its closest relative is Mofidra (the same fp32 stream,
+parallel sublayers and attention kernels).
+
 Rooflines: 2.5 PFLOP/s dense bf16 MFMA, 8 TB/s HBM.  A kernel's ``roof_frac`` is
-max(flops / peak, bytes / bandwidth) / measured time.
+max(flops / peak, bytes / bandwidth) / measured time.  The recurrence runs on the vector ALUs:
+its compute roof is 157 TFLOP/s fp32.
 """
 
 import json
@@ -16,12 +24,14 @@ import time
 
 import torch
 
-from ..models.config import MofidraConfig, ModelConfig
+from ..models.config import MofidraConfig, ModelConfig, PadadraConfig
 from ..models.mofidra import MofidraModel
+from ..models.padadra import PadadraModel
 from ..models.transformer import AttnMeta, DecoderModel
 from ..ops import get_ops
 
 PEAK_FLOPS, PEAK_BW = 2.5e15, 8.0e12
+PEAK_VALU = 157e12
 BS = 16
 
 SIZES = {
@@ -39,6 +49,20 @@ def mofidra_config(s, moe: bool) -> MofidraConfig:
                                     "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
                                     "layers": [{"type": "attention", "mixer": mixer, "mlp": mlp}] * s["layers"]},
                                    "mofidra-bench")
+
+
+def padadra_config(s) -> PadadraConfig:
+    H, G = s["heads"], s["kv_heads"]
+    left = {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128, "scale": 0.088, "conv": 4, "mask": {"size": 512},
+            "rot": {"dims": 64, "base": 1e6, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    par = {"type": "parallel", "mixer": {"left": left, "right": {"heads": H // 2, "dim": 64, "vdim": 128}},
+           "mlp": {"kind": "dense", "ff": s["ff"]}}
+    delta = {"type": "channel_delta", "mixer": {"heads": H, "kv_heads": H // 2, "dim": 128, "vdim": 128, "conv": 4,
+                                                "decay_rank": 64, "gate_rank": 64}, "mlp": {"kind": "dense", "ff": s["ff"]}}
+    layers = [delta if i % 4 == 1 else par for i in range(s["layers"])]
+    return PadadraConfig.from_dict({"architecture": "Padadra", "width": s["width"], "vocab": s["vocab"],
+                                    "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 31}},
+                                    "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": layers}, "padadra-bench")
 
 
 def decoder_config(s) -> ModelConfig:
@@ -67,7 +91,8 @@ def step_meta(n_seq, ctx, q_len, tile_rows, device, split_single):
                     max_q_len=q_len, decode=decode, tile_rows=tile_rows,
                     logits_idx=(q_start[1:] - 1).long().to(device),
                     tiles=torch.tensor([t[1:] for t in tiles], dtype=i32, device=device).reshape(-1, 3),
-                    single=torch.zeros(0, 2, dtype=i32, device=device) if split_single else None)
+                    single=torch.zeros(0, 2, dtype=i32, device=device) if split_single else None,
+                    token_seq=seq.to(i32).to(device), state_rows=torch.arange(n_seq, dtype=i32, device=device))
     return meta, n_seq * nblk + 1
 
 
@@ -104,12 +129,15 @@ def model_throughput(model, prefill=(8, 1024), decode=(64, 1024)):
     meta, nb = step_meta(n, s, s, tile_rows, dev, split)
     k, v = model.alloc_kv(max(nb, decode[0] * ((decode[1] + BS - 1) // BS) + 1), BS, torch.bfloat16)
     tokens = torch.randint(0, model.cfg.vocab_size, (n * s,), dtype=torch.int32, device=dev)
+    state = model.alloc_state(max(n, decode[0]) + 1) if hasattr(model, "alloc_state") else None
+    meta.state = state
     t = _time(lambda: model.forward(tokens, meta, k, v), iters=5)
     out["prefill_tokens_per_s"] = round(n * s / t)
     out["prefill_ms"] = round(t * 1e3, 3)
     b, ctx = decode
     dmeta, _ = step_meta(b, ctx, 1, tile_rows, dev, split)
     dmeta.logits_idx = None
+    dmeta.state = state
     dtok = torch.randint(0, model.cfg.vocab_size, (b,), dtype=torch.int32, device=dev)
     t = _graph_time(lambda: model.forward(dtok, dmeta, k, v))
     out["decode_tokens_per_s"] = round(b / t)
@@ -185,6 +213,84 @@ def kernel_pairs(s, dev):
     return out
 
 
+def state_kernels(s, dev):
+    """The Padadra kernels beside their like kernels of Mofidra at the same shapes (window + sink
+    attention: the two-map attention; scalar-gain residual kernel: the weighted one; pair rotary
+    with norms: the half-split rotary), and the kernels without a relative (recurrence, convolution)."""
+    ops = get_ops("hip")
+    H, G, W = s["heads"], s["kv_heads"], s["width"]
+    bf = torch.bfloat16
+    out = {}
+    n, ctx, window = 8, 1024, 512
+    T = n * ctx
+    # ---- prefill attention, 8 x 1024: one 128-wide map, 512-key window, sink ----
+    pairs = sum(min(i + 1, window) for i in range(ctx)) * n
+    flops = 2 * H * 256 * pairs
+    io = T * H * 256 * 2 + T * G * 256 * 2
+    meta, nb = step_meta(n, ctx, ctx, 64, dev, True)
+    q = torch.randn(T, H, 128, device=dev, dtype=bf)
+    kc, vc = torch.randn(nb, G, BS, 128, device=dev, dtype=bf), torch.randn(nb, G, 128, BS, device=dev, dtype=bf)
+    sink = torch.randn(H, device=dev)
+    t = _time(lambda: ops.multimap_attention(q, kc, vc, meta, 0.088, 1, 0.0, -1.0, 1.0, 128, window, sink))
+    out["prefill_attention"] = {"padadra_ms": round(t * 1e3, 3), "padadra_roof_frac": _roof(flops, io, t)}
+    q2 = torch.randn(T, H, 128, device=dev, dtype=bf)
+    t = _time(lambda: ops.multimap_attention(q2, kc, vc, meta, 0.125, 2, 0.4, 1e-5, 0.5, 128))
+    full = 2 * H * 256 * n * ctx * ctx / 2
+    out["prefill_attention"].update({"mofidra_ms": round(t * 1e3, 3), "mofidra_roof_frac": _roof(1.5 * full, io, t)})
+    # ---- decode attention, 64 rows x 1024 context ----
+    b = 64
+    dmeta, nb = step_meta(b, ctx, 1, 64, dev, True)
+    kc, vc = torch.randn(nb, G, BS, 128, device=dev, dtype=bf), torch.randn(nb, G, 128, BS, device=dev, dtype=bf)
+    qd = torch.randn(b, H, 128, device=dev, dtype=bf)
+    t = _graph_time(lambda: ops.multimap_attention(qd, kc, vc, dmeta, 0.088, 1, 0.0, -1.0, 1.0, 128, window, sink), iters=50)
+    out["decode_attention"] = {"padadra_ms": round(t * 1e3, 4),
+                               "padadra_roof_frac": _roof(2 * H * 256 * b * window, b * window * G * 256 * 2, t)}
+    t = _graph_time(lambda: ops.multimap_attention(qd, kc, vc, dmeta, 0.125, 2, 0.4, 1e-5, 0.5, 128), iters=50)
+    out["decode_attention"].update({"mofidra_ms": round(t * 1e3, 4),
+                                    "mofidra_roof_frac": _roof(2 * H * 256 * b * ctx * 1.5, b * ctx * G * 256 * 2, t)})
+    # ---- residual update + next norms, 8192 rows ----
+    x32 = torch.randn(T, W, device=dev)
+    a, c, p = (torch.randn(T, W, device=dev, dtype=bf) for _ in range(3))
+    wa, wb = torch.randn(W, device=dev), torch.randn(W, device=dev)
+    t = _time(lambda: ops.residual_mix_norm(x32, [(a, wa), (c, wb)], 0.5, [p], 0.5, 1e-5, (1.0, 0.9), bf), iters=20)
+    out["residual_norm"] = {"padadra_ms": round(t * 1e3, 4), "padadra_roof_frac": _roof(0, T * W * (4 + 4 + 3 * 2 + 2 * 2), t)}
+    w32 = torch.zeros(W, device=dev)
+    t = _time(lambda: ops.residual_add_rmsnorm32(x32, [a, p], w32, 1e-5, 1.0, bf), iters=20)
+    out["residual_norm"].update({"mofidra_ms": round(t * 1e3, 4), "mofidra_roof_frac": _roof(0, T * W * (4 + 4 + 2 + 2 + 2), t)})
+    # ---- rotary + cache write, 8192 rows ----
+    width = (H + G) * 128 + G * 128
+    y = torch.randn(T, width, device=dev, dtype=bf)
+    qn, kn = torch.ones(H * 128, device=dev), torch.ones(G * 128, device=dev)
+    inv, vinv = torch.rand(32, device=dev), torch.rand(64, device=dev)
+    kc, vc = torch.zeros(n * ctx // BS + 1, G, BS, 128, device=dev, dtype=bf), torch.zeros(n * ctx // BS + 1, G, 128, BS, device=dev, dtype=bf)
+    t = _time(lambda: ops.rope_pairs_kv_write(y, meta.positions, meta.slots, H, G, 128, 128, qn, kn, 1e-5, inv, vinv, kc, vc), iters=20)
+    io = T * width * 2 * 2
+    out["rotary_kv_write"] = {"padadra_ms": round(t * 1e3, 4), "padadra_roof_frac": _roof(0, io, t)}
+    kc2 = torch.zeros(n * ctx // BS + 1, G, BS, 128, device=dev, dtype=bf)
+    t = _time(lambda: ops.rope_multi_kv_write(y, meta.positions, meta.slots, H, G, 2, 64, 128, inv, kc2, vc), iters=20)
+    out["rotary_kv_write"].update({"mofidra_ms": round(t * 1e3, 4), "mofidra_roof_frac": _roof(0, io, t)})
+    # ---- short convolution, 8192 rows ----
+    cw = torch.randn(width, 4, device=dev)
+    cstate = torch.zeros(n + 1, 3, width, device=dev, dtype=bf)
+    t = _time(lambda: ops.short_conv(y, width, cw, meta, cstate, "silu"), iters=20)
+    out["short_conv"] = {"padadra_ms": round(t * 1e3, 4), "padadra_roof_frac": _roof(0, io, t)}
+    # ---- the recurrence: gated delta rule, H heads of 128 x 128 state ----
+    Gq = max(1, H // 2)
+    for name, rows_, m_ in (("prefill", T, meta), ("decode", b, dmeta)):
+        q32, k32 = torch.randn(rows_, Gq, 128, device=dev) * 0.1, torch.randn(rows_, Gq, 128, device=dev) * 0.1
+        g32, beta = torch.rand(rows_, H, 128, device=dev), torch.rand(rows_, H, device=dev)
+        v = torch.randn(rows_, H * 128, device=dev, dtype=bf)
+        S = torch.zeros(max(n, b) + 1, H, 128, 128, device=dev)
+        m_.state_rows = torch.arange(m_.q_start.numel() - 1, dtype=torch.int32, device=dev)
+        fn = lambda: ops.gated_state_scan(q32, k32, g32, v, beta, m_, S, True)  # noqa: E731
+        t = _time(fn, iters=10) if name == "prefill" else _graph_time(fn, iters=50)
+        flops = rows_ * H * 128 * 128 * 8
+        io = rows_ * (2 * Gq * 128 * 4 + H * 128 * 4 + H * 128 * 2 + H * 128 * 4) + (m_.q_start.numel() - 1) * H * 128 * 128 * 4 * 2
+        out[f"state_scan_{name}"] = {"padadra_ms": round(t * 1e3, 4),
+                                     "padadra_roof_frac": round(max(flops / PEAK_VALU, io / PEAK_BW) / t, 4)}
+    return out
+
+
 def run(sizes=("w2048", "w4096"), kernels=True) -> dict:
     dev = torch.device("cuda", torch.cuda.current_device())
     ops = get_ops("hip")
@@ -196,6 +302,7 @@ def run(sizes=("w2048", "w4096"), kernels=True) -> dict:
             entry = {}
             for label, build in (("mofidra_dense", lambda: MofidraModel(mofidra_config(s, False), ops, dev)),
                                  ("mofidra_moe", lambda: MofidraModel(mofidra_config(s, True), ops, dev)),
+                                 ("padadra", lambda: PadadraModel(padadra_config(s), ops, dev)),
                                  ("decoder", lambda: DecoderModel(decoder_config(s), ops, dev))):
                 model = build()
                 model.init_random(seed=1, std=0.02)
@@ -204,6 +311,7 @@ def run(sizes=("w2048", "w4096"), kernels=True) -> dict:
                 torch.cuda.empty_cache()
             if kernels:
                 entry["kernels"] = kernel_pairs(s, dev)
+                entry["state_kernels"] = state_kernels(s, dev)
             result["sizes"][name] = entry
     return result
 
