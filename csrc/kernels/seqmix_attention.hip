@@ -68,13 +68,13 @@ struct AttnArgs {
 // Everything that does not depend on the lane stays scalar: the page lookup and the slab base go
 // to SGPRs, a lane adds a 32-bit offset that is fixed for the whole loop.  Scores are kept in the
 // log2 domain (scale * log2 e folded into one multiply, v_exp_f32 directly).
-template <typename T, int KC, int VT, int KT, bool PF, bool FULL, bool EXACT>
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int EXACT>
 __device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const typename Elem<T>::frag (&qf)[2][KC],
                                              int limit, int limit_min, int lo, int lo_max, int k_begin, int k_last,
                                              const int* __restrict__ table, f32x4 (&acc)[2][VT], float (&mx)[2],
                                              float (&den)[2]) {
   typedef typename Elem<T>::frag F;
-  // EXACT: two maps, dim = 16 KC, vdim = 16 VT, 16-token pages, fragment-major slabs -- every guard
+  // EXACT (1 or 2 = the number of maps): dim = 16 KC, vdim = 16 VT, 16-token pages, fragment-major slabs -- every guard
   // below is a compile-time constant, fragment offsets are immediates, the loop body is straight-line
   struct Shape {
     const AttnArgs& r;
@@ -82,7 +82,7 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const ty
     float scale;
     const void *k_cache, *v_cache;
   };
-  const Shape a{a_, EXACT ? 2 : a_.maps, EXACT ? 16 * KC : a_.dim, EXACT ? 16 * VT : a_.vdim, EXACT ? 1 : a_.swz, EXACT ? 16 : a_.BS, a_.G,
+  const Shape a{a_, EXACT ? EXACT : a_.maps, EXACT ? 16 * KC : a_.dim, EXACT ? 16 * VT : a_.vdim, EXACT ? 1 : a_.swz, EXACT ? 16 : a_.BS, a_.G,
                 a_.max_blocks, a_.num_blocks, EXACT ? 1 : a_.vec_k, EXACT ? 1 : a_.vec_v, a_.scale, a_.k_cache, a_.v_cache};
   const int lane = threadIdx.x & 63, col = lane & 15, grp = lane >> 4;
   const int KD = a.maps * a.dim;
@@ -226,7 +226,7 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const ty
   }
 }
 
-template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC, bool EXACT = false>
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC, int EXACT = 0>
 __global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
   typedef typename Elem<T>::frag F;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -301,7 +301,7 @@ __global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
 // head g (H / G) + 16 cg + c of the same token, so K and V^T are read once per KV head.  One wave
 // per (item, KV head x column group, SPLIT_KEYS-key split); partials as the merge kernel reads them
 // (running maxima in the log2 domain of `attend_range`).
-template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC, bool EXACT = false>
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC, int EXACT = 0>
 __global__ __launch_bounds__(64, OCC) void decode_mfma_kernel(AttnArgs a) {
   typedef typename Elem<T>::frag F;
   const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
@@ -410,11 +410,20 @@ int launch_prefill(const AttnArgs& a, int n_tiles, int tile_rows, hipStream_t s)
   const bool small = a.dim <= 64 && a.vdim <= 128;
   const bool full = a.dim % 16 == 0 && a.vdim % 16 == 0 && a.vec_k && a.vec_v;   // whole, aligned fragments only
   if (tile_rows != 64) return -2;
+  if constexpr (sizeof(T) == 2) if (full && a.maps == 1 && a.swz && a.BS == 16) {   // one-map heads, exact shapes
+#define BCG_EXACT1(KC_, VT_)                                                                     \
+  if (a.dim == 16 * KC_ && a.vdim == 16 * VT_) {                                                 \
+    prefill_kernel<T, KC_, VT_, 2, true, true, 2, 1><<<grid, 256, 0, s>>>(a);                    \
+    return BCG_CHECK_LAUNCH();                                                                   \
+  }
+    BCG_EXACT1(8, 8) BCG_EXACT1(4, 4) BCG_EXACT1(4, 8) BCG_EXACT1(2, 2) BCG_EXACT1(6, 6)
+#undef BCG_EXACT1
+  }
   if constexpr (sizeof(T) == 2) if (small) {
     const bool exact = full && a.maps == 2 && a.swz && a.BS == 16;
 #define BCG_EXACT(KC_, VT_)                                                                      \
   if (exact && a.dim == 16 * KC_ && a.vdim == 16 * VT_) {                                        \
-    prefill_kernel<T, KC_, VT_, 2, true, true, 2, true><<<grid, 256, 0, s>>>(a);                 \
+    prefill_kernel<T, KC_, VT_, 2, true, true, 2, 2><<<grid, 256, 0, s>>>(a);                    \
     return BCG_CHECK_LAUNCH();                                                                   \
   }
     BCG_EXACT(4, 8) BCG_EXACT(3, 6) BCG_EXACT(2, 4) BCG_EXACT(4, 4) BCG_EXACT(2, 2)
@@ -438,14 +447,23 @@ int launch_decode(const AttnArgs& a, int n_items, hipStream_t s) {
   dim3 grid(a.G * ((per + 15) / 16), a.n_splits, n_items);
   const bool full = a.dim % 16 == 0 && a.vdim % 16 == 0 && a.vec_k && a.vec_v;
   bool done = false;
-  if constexpr (sizeof(T) == 2) if (a.dim <= 64 && a.vdim <= 128) {
+  if constexpr (sizeof(T) == 2) if (full && a.maps == 1 && a.swz && a.BS == 16) {   // one-map heads, exact shapes
+#define BCG_EXACT1(KC_, VT_)                                                                     \
+  if (!done && a.dim == 16 * KC_ && a.vdim == 16 * VT_) {                                        \
+    done = true;                                                                                 \
+    decode_mfma_kernel<T, KC_, VT_, 2, true, true, 2, 1><<<grid, 64, 0, s>>>(a);                 \
+  }
+    BCG_EXACT1(8, 8) BCG_EXACT1(4, 4) BCG_EXACT1(4, 8) BCG_EXACT1(2, 2) BCG_EXACT1(6, 6)
+#undef BCG_EXACT1
+  }
+  if constexpr (sizeof(T) == 2) if (!done && a.dim <= 64 && a.vdim <= 128) {
     done = true;
     const bool exact = full && a.maps == 2 && a.swz && a.BS == 16;
     bool hit = false;
 #define BCG_EXACT(KC_, VT_)                                                                      \
   if (!hit && exact && a.dim == 16 * KC_ && a.vdim == 16 * VT_) {                                \
     hit = true;                                                                                  \
-    decode_mfma_kernel<T, KC_, VT_, 2, true, true, 2, true><<<grid, 64, 0, s>>>(a);              \
+    decode_mfma_kernel<T, KC_, VT_, 2, true, true, 2, 2><<<grid, 64, 0, s>>>(a);                 \
   }
     BCG_EXACT(4, 8) BCG_EXACT(3, 6) BCG_EXACT(2, 4) BCG_EXACT(4, 4) BCG_EXACT(2, 2)
 #undef BCG_EXACT

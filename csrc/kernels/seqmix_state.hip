@@ -165,6 +165,68 @@ __global__ __launch_bounds__(NT) void short_conv_kernel(const T* __restrict__ y,
   out[static_cast<size_t>(t) * C + c] = Elem<T>::st(acc);
 }
 
+// The same for VEC consecutive channels per thread (one 16-byte load per tap) and CONV_ROWS
+// consecutive rows per block, the thread's TAPS x VEC weights in registers.  Needs C, the row
+// strides and the base addresses to be multiples of VEC elements.
+constexpr int CONV_ROWS = 8;
+
+template <typename T, int VEC, int TAPS>
+__global__ __launch_bounds__(NT) void short_conv_vec_kernel(const T* __restrict__ y, int64_t y_stride, int C,
+                                                            const float* __restrict__ w, const int* __restrict__ positions,
+                                                            const int* __restrict__ token_seq, const int* __restrict__ q_start,
+                                                            const int* __restrict__ state_rows, const T* __restrict__ state,
+                                                            int n_rows, T* __restrict__ out, int act, int T_) {
+  struct alignas(sizeof(T) * VEC) Vec { T e[VEC]; };
+  const int c = (blockIdx.y * NT + threadIdx.x) * VEC;
+  if (c >= C) return;
+  float wr[VEC][TAPS];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e)
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) wr[e][j] = w[static_cast<size_t>(c + e) * TAPS + j];
+  const int t_end = min(T_, (static_cast<int>(blockIdx.x) + 1) * CONV_ROWS);
+  for (int t = blockIdx.x * CONV_ROWS; t < t_end; ++t) {
+    const int seg = token_seq[t], off = t - q_start[seg], pos = positions[t];
+    const int sr = state_rows[seg];
+    const bool row_ok = sr >= 0 && sr < n_rows;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) {
+      const int back = TAPS - 1 - j;
+      const T* src = nullptr;
+      if (off >= back) src = y + static_cast<size_t>(t - back) * y_stride + c;
+      else if (pos - back >= 0 && row_ok) src = state + (static_cast<size_t>(sr) * (TAPS - 1) + (j + off)) * C + c;
+      if (src != nullptr) {
+        const Vec u = *reinterpret_cast<const Vec*>(src);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] += wr[e][j] * Elem<T>::ld(u.e[e]);
+      }
+    }
+    Vec o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float v = act == 1 ? acc[e] * sigmoidf_(acc[e]) : acc[e];
+      o.e[e] = Elem<T>::st(v);
+    }
+    *reinterpret_cast<Vec*>(out + static_cast<size_t>(t) * C + c) = o;
+  }
+}
+
+template <typename T>
+bool launch_conv_vec(const T* y, int64_t y_stride, int C, const float* w, int taps, const int* ps, const int* ts, const int* qs,
+                     const int* sr, const T* state, int n_rows, T* out, int act, int T_, hipStream_t s) {
+  constexpr int VEC = 16 / sizeof(T);
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(state) | reinterpret_cast<uintptr_t>(out);
+  if (C % VEC || y_stride % VEC || bits % 16 || taps < 2 || taps > 4) return false;
+  dim3 grid((T_ + CONV_ROWS - 1) / CONV_ROWS, (C / VEC + NT - 1) / NT);
+  if (taps == 2) short_conv_vec_kernel<T, VEC, 2><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_);
+  else if (taps == 3) short_conv_vec_kernel<T, VEC, 3><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_);
+  else short_conv_vec_kernel<T, VEC, 4><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_);
+  return true;
+}
+
 // The state row after the segment: its last taps - 1 inputs (older ones move up from the old state).
 template <typename T>
 __global__ __launch_bounds__(NT) void short_conv_state_kernel(const T* __restrict__ y, int64_t y_stride, int C, int taps,
@@ -525,6 +587,11 @@ BCG_API int bcg_short_conv(const void* y, int64_t y_stride, int C, const void* w
   const float* wf = static_cast<const float*>(w);
   dim3 grid(T_, (C + NT - 1) / NT), sgrid(B, (C + NT - 1) / NT);
   if (T_ > 2147483647 / 2 || grid.y > 65535) return -2;
+  const bool vec = is_f32 ? launch_conv_vec<float>(static_cast<const float*>(y), y_stride, C, wf, taps, ps, ts, qs, sr,
+                                                   static_cast<const float*>(state), n_rows, static_cast<float*>(out), act, T_, s)
+                          : launch_conv_vec<bf16_t>(static_cast<const bf16_t*>(y), y_stride, C, wf, taps, ps, ts, qs, sr,
+                                                    static_cast<const bf16_t*>(state), n_rows, static_cast<bf16_t*>(out), act, T_, s);
+  if (!vec)
   BCG_BY_TYPE((short_conv_kernel<float><<<grid, NT, 0, s>>>(static_cast<const float*>(y), y_stride, C, wf, taps, ps, ts, qs, sr,
                                                            static_cast<const float*>(state), n_rows, static_cast<float*>(out), act)),
               (short_conv_kernel<bf16_t><<<grid, NT, 0, s>>>(static_cast<const bf16_t*>(y), y_stride, C, wf, taps, ps, ts, qs, sr,

@@ -66,12 +66,14 @@ def test_residual_mix_norm(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("taps,act", [(4, None), (2, "silu"), (7, None), (1, "silu")])
-def test_short_conv_and_its_state(ops, dtype, taps, act):
+@pytest.mark.parametrize("taps,act,Cn,pad", [(4, None, 300, 11), (2, "silu", 304, 8), (7, None, 300, 11), (1, "silu", 300, 11),
+                                             (3, None, 512, 0), (4, "silu", 2056, 8)])
+def test_short_conv_and_its_state(ops, dtype, taps, act, Cn, pad):
+    """Widths and strides on and off the 16-byte grid (vector and element kernels)."""
     g = torch.Generator().manual_seed(taps)
     mc, md = _meta(PARTS, ROWS)
-    T, Cn = mc.positions.numel(), 300
-    y = torch.randn(T, Cn + 11, generator=g).to(dtype)
+    T = mc.positions.numel()
+    y = torch.randn(T, Cn + pad, generator=g).to(dtype)
     w = torch.randn(Cn, taps, generator=g)
     state = torch.randn(6, taps - 1, Cn, generator=g).to(dtype) if taps > 1 else None
     sd = state.to(DEV) if taps > 1 else None
@@ -135,7 +137,8 @@ def _attention_inputs(H, G, d, e, lens, q_lens, dtype, seed, loud=None):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,d,e", [(8, 1, 64, 64), (4, 2, 16, 24), (6, 2, 72, 40), (34, 2, 32, 32)])
+@pytest.mark.parametrize("H,G,d,e", [(8, 1, 64, 64), (4, 2, 16, 24), (6, 2, 72, 40), (34, 2, 32, 32), (4, 2, 128, 128),
+                                     (2, 1, 64, 128), (3, 1, 96, 96)])
 @pytest.mark.parametrize("window", [0, 1, 16, 37, 96, 400])
 def test_window_and_sink_attention(ops, dtype, H, G, d, e, window):
     """Prefill tiles and single rows in one step; the loud key sits just outside the last query's
