@@ -19,6 +19,8 @@ namespace {
 
 constexpr int NT = 256;
 constexpr int MAX_TAPS = 16;
+constexpr int SCAN_CHUNK = 4;
+constexpr int SCAN_WAVES = 4;   // waves of a recurrence workgroup (8 value columns each)   // tokens of a recurrence staged through LDS at a time
 
 __device__ __forceinline__ float block_sum(float v, float* red) {
   v = wave_sum(v);
@@ -410,10 +412,14 @@ __global__ __launch_bounds__(NT) void delta_prepare_kernel(const T* __restrict__
 // ---------------------------------------------------------------- the recurrence
 // Per head a dim x vdim fp32 state S; token after token
 //     S <- diag(g_t) S;  u = DELTA ? beta_t (v_t - S^T k_t) : v_t;  S <- S + k_t u^T;  o_t = S^T q_t.
-// One wave per (segment, head, 64 value columns): a lane owns one column of S in registers, so
-// no lane ever waits for another.  The token's q / k / g vectors are loaded one element per lane
-// and broadcast from there (v_readlane with a constant lane: the operand of the multiply-add is
-// an SGPR); the next token's vectors are loaded while this one's are used.
+// One workgroup of SCAN_WAVES waves per (segment, head, 8 SCAN_WAVES value columns); a wave owns 8
+// columns: lane = 8 column + row group, so a lane keeps
+// dim / 8 rows of one column of S in registers and the two sums over rows (S^T k and S^T q) are
+// finished inside a group of 8 neighbouring lanes with three DPP adds (no LDS round trip).  The
+// tokens' q / k / g vectors are staged through LDS SCAN_CHUNK tokens at a time (every lane reads
+// its row group's 16-byte pieces; the groups' pieces are padded apart so that they fall into
+// different banks) by the whole workgroup, so a head's vectors are fetched once per 8 SCAN_WAVES
+// columns; the next chunk's loads fly under this chunk's arithmetic.
 struct ScanArgs {
   const float* q; const float* k; const float* g;   // [T, Gq, dim], [T, Gq, dim], [T, H, dim]
   const void* v; int64_t v_stride;                  // [T, >= H vdim]
@@ -424,76 +430,126 @@ struct ScanArgs {
   int n_rows, H, Gq, dim, vdim;
 };
 
-__device__ __forceinline__ float bcast(float v, int lane) {
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+  return x + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
+// sum over the 8 lanes of a group (lanes 8n .. 8n + 7), the result in every lane of the group:
+// neighbours in a quad, the quad's other pair, then the mirror lane of the other quad
+__device__ __forceinline__ float group8_sum(float x) {
+  x = dpp_add<0xB1>(x);    // quad_perm [1, 0, 3, 2]
+  x = dpp_add<0x4E>(x);    // quad_perm [2, 3, 0, 1]
+  return dpp_add<0x141>(x);  // row_half_mirror
 }
 
 template <typename T, int DMAX, bool DELTA>
-__global__ __launch_bounds__(64) void state_scan_kernel(ScanArgs a) {
-  constexpr int NV = (DMAX + 63) / 64;
-  const int lane = threadIdx.x, b = blockIdx.x, h = blockIdx.y, j = blockIdx.z * 64 + lane;
+__global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a) {
+  constexpr int RPL = DMAX / 8;                      // rows per lane
+  constexpr int GP = RPL + 4;                        // a row group's piece of a staged vector, padded
+  constexpr int VP = 8 * GP;                         // one staged vector
+  constexpr int NTH = 64 * SCAN_WAVES;
+  constexpr int NL = (3 * DMAX + NTH - 1) / NTH;     // staged elements per thread and token: q | k | g
+  constexpr int CT = SCAN_CHUNK;                     // tokens staged at a time
+  __shared__ __attribute__((aligned(16))) float vec[2][CT][3 * VP];
+  const int tid = threadIdx.x, lane = tid & 63, col = lane >> 3, rg = lane & 7;
+  const int b = blockIdx.x, h = blockIdx.y, j = (blockIdx.z * SCAN_WAVES + (tid >> 6)) * 8 + col;
   const int t0 = a.q_start[b], t1 = a.q_start[b + 1];
   const int sr = a.state_rows[b];
   if (t1 <= t0 || sr < 0 || sr >= a.n_rows) return;
   const bool col_ok = j < a.vdim;
   const int gq = h / (a.H / a.Gq);
   const int dim = a.dim, vdim = a.vdim;
-  float* Sp = a.state + (static_cast<size_t>(sr) * a.H + h) * dim * vdim + (col_ok ? j : 0);
+  float* Sp = a.state + ((static_cast<size_t>(sr) * a.H + h) * dim + rg * RPL) * vdim + (col_ok ? j : 0);
   const bool load_state = a.positions[t0] != 0 && col_ok;
-  float S[DMAX];
+  float S[RPL];
 #pragma unroll
-  for (int i = 0; i < DMAX; ++i) S[i] = (load_state && i < dim) ? Sp[static_cast<size_t>(i) * vdim] : 0.f;
+  for (int i = 0; i < RPL; ++i) S[i] = (load_state && rg * RPL + i < dim) ? Sp[static_cast<size_t>(i) * vdim] : 0.f;
   const T* vbase = static_cast<const T*>(a.v) + h * vdim + (col_ok ? j : 0);
 
-  float qv[NV], kv[NV], gv[NV], vv, bt = 1.0f;
-  auto load = [&](int t, float (&q)[NV], float (&k)[NV], float (&g)[NV], float& v, float& be) {
-    const float* qp = a.q + (static_cast<size_t>(t) * a.Gq + gq) * dim;
-    const float* kp = a.k + (static_cast<size_t>(t) * a.Gq + gq) * dim;
-    const float* gp = a.g + (static_cast<size_t>(t) * a.H + h) * dim;
+  // element e of a token is (which of q, k, g; row); rows past dim are zero
+  struct Chunk { float r[CT][NL], v[CT], be[CT]; };
+  auto load = [&](int first, Chunk& c) {
 #pragma unroll
-    for (int n = 0; n < NV; ++n) {
-      const int i = lane + 64 * n;
-      const bool ok = i < dim;             // rows past dim: k = g = q = 0, the state rows stay zero
-      q[n] = ok ? qp[i] : 0.f;
-      k[n] = ok ? kp[i] : 0.f;
-      g[n] = ok ? gp[i] : 0.f;
-    }
-    v = col_ok ? Elem<T>::ld(vbase[static_cast<size_t>(t) * a.v_stride]) : 0.f;
-    if (DELTA) be = a.beta[static_cast<size_t>(t) * a.H + h];
-  };
-  load(t0, qv, kv, gv, vv, bt);
-  for (int t = t0; t < t1; ++t) {
-    float qn[NV], kn[NV], gn[NV], vn = 0.f, bn = 1.0f;
+    for (int tt = 0; tt < CT; ++tt) {
+      const int t = first + tt;
+      const bool live = t < t1;
 #pragma unroll
-    for (int n = 0; n < NV; ++n) qn[n] = kn[n] = gn[n] = 0.f;
-    if (t + 1 < t1) load(t + 1, qn, kn, gn, vn, bn);
-    float u = vv;
-    if (DELTA) {
-      float d[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int i = 0; i < DMAX; ++i) {
-        S[i] *= bcast(gv[i >> 6], i & 63);
-        d[i & 3] += S[i] * bcast(kv[i >> 6], i & 63);
+      for (int n = 0; n < NL; ++n) {
+        const int e = tid + NTH * n, which = e / DMAX, i = e - which * DMAX;
+        const float* p = which == 0 ? a.q + (static_cast<size_t>(t) * a.Gq + gq) * dim
+                       : which == 1 ? a.k + (static_cast<size_t>(t) * a.Gq + gq) * dim
+                                    : a.g + (static_cast<size_t>(t) * a.H + h) * dim;
+        c.r[tt][n] = (live && which < 3 && i < dim) ? p[i] : 0.f;
       }
-      u = bt * (vv - ((d[0] + d[1]) + (d[2] + d[3])));
+      c.v[tt] = (live && col_ok) ? Elem<T>::ld(vbase[static_cast<size_t>(t) * a.v_stride]) : 0.f;
+      c.be[tt] = (DELTA && live) ? a.beta[static_cast<size_t>(t) * a.H + h] : 1.0f;
     }
-    float o[4] = {0.f, 0.f, 0.f, 0.f};
+  };
+  auto stage = [&](int buf, const Chunk& c) {
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i) {
-      const float ki = bcast(kv[i >> 6], i & 63);
-      if (DELTA) S[i] += ki * u;
-      else S[i] = S[i] * bcast(gv[i >> 6], i & 63) + ki * u;
-      o[i & 3] += S[i] * bcast(qv[i >> 6], i & 63);
+    for (int tt = 0; tt < CT; ++tt)
+#pragma unroll
+      for (int n = 0; n < NL; ++n) {
+        const int e = tid + NTH * n, which = e / DMAX, i = e - which * DMAX;
+        if (e < 3 * DMAX) vec[buf][tt][which * VP + (i / RPL) * GP + (i % RPL)] = c.r[tt][n];
+      }
+  };
+  Chunk cur, nxt;
+  load(t0, cur);
+  stage(0, cur);
+  __syncthreads();
+  int buf = 0;
+  for (int first = t0; first < t1; first += CT, buf ^= 1) {
+    const bool more = first + CT < t1;
+    if (more) load(first + CT, nxt);
+#pragma unroll
+    for (int tt = 0; tt < CT; ++tt) {
+      const int t = first + tt;
+      if (t < t1) {
+        const f32x4* qv = reinterpret_cast<const f32x4*>(&vec[buf][tt][rg * GP]);
+        const f32x4* kv = reinterpret_cast<const f32x4*>(&vec[buf][tt][VP + rg * GP]);
+        const f32x4* gv = reinterpret_cast<const f32x4*>(&vec[buf][tt][2 * VP + rg * GP]);
+        float u = cur.v[tt];
+        if (DELTA) {
+          float d[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int m = 0; m < RPL / 4; ++m) {
+            const f32x4 g4 = gv[m], k4 = kv[m];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              S[4 * m + i] *= g4[i];
+              d[i] += S[4 * m + i] * k4[i];
+            }
+          }
+          u = cur.be[tt] * (u - group8_sum((d[0] + d[1]) + (d[2] + d[3])));
+        }
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int m = 0; m < RPL / 4; ++m) {
+          const f32x4 k4 = kv[m], q4 = qv[m];
+          f32x4 g4 = {1.f, 1.f, 1.f, 1.f};
+          if (!DELTA) g4 = gv[m];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (DELTA) S[4 * m + i] += k4[i] * u;
+            else S[4 * m + i] = S[4 * m + i] * g4[i] + k4[i] * u;
+            o[i] += S[4 * m + i] * q4[i];
+          }
+        }
+        const float os = group8_sum((o[0] + o[1]) + (o[2] + o[3]));
+        if (col_ok && rg == 0) a.out[(static_cast<size_t>(t) * a.H + h) * vdim + j] = os;
+      }
     }
-    if (col_ok) a.out[(static_cast<size_t>(t) * a.H + h) * vdim + j] = (o[0] + o[1]) + (o[2] + o[3]);
-#pragma unroll
-    for (int n = 0; n < NV; ++n) { qv[n] = qn[n]; kv[n] = kn[n]; gv[n] = gn[n]; }
-    vv = vn; bt = bn;
+    if (more) {
+      stage(buf ^ 1, nxt);   // (the other buffer: its readers finished before the last barrier)
+      cur = nxt;
+    }
+    __syncthreads();
   }
   if (col_ok) {
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i)
-      if (i < dim) Sp[static_cast<size_t>(i) * vdim] = S[i];
+    for (int i = 0; i < RPL; ++i)
+      if (rg * RPL + i < dim) Sp[static_cast<size_t>(i) * vdim] = S[i];
   }
 }
 
@@ -521,11 +577,10 @@ __global__ __launch_bounds__(NT) void head_norm_gate_kernel(const float* __restr
 
 template <typename T, bool DELTA>
 int launch_scan(const ScanArgs& a, int B, hipStream_t s) {
-  dim3 grid(B, a.H, (a.vdim + 63) / 64);
-  if (a.dim <= 16) state_scan_kernel<T, 16, DELTA><<<grid, 64, 0, s>>>(a);
-  else if (a.dim <= 32) state_scan_kernel<T, 32, DELTA><<<grid, 64, 0, s>>>(a);
-  else if (a.dim <= 64) state_scan_kernel<T, 64, DELTA><<<grid, 64, 0, s>>>(a);
-  else state_scan_kernel<T, 128, DELTA><<<grid, 64, 0, s>>>(a);
+  dim3 grid(B, a.H, (a.vdim + 8 * SCAN_WAVES - 1) / (8 * SCAN_WAVES));
+  if (a.dim <= 32) state_scan_kernel<T, 32, DELTA><<<grid, 64 * SCAN_WAVES, 0, s>>>(a);
+  else if (a.dim <= 64) state_scan_kernel<T, 64, DELTA><<<grid, 64 * SCAN_WAVES, 0, s>>>(a);
+  else state_scan_kernel<T, 128, DELTA><<<grid, 64 * SCAN_WAVES, 0, s>>>(a);
   return BCG_CHECK_LAUNCH();
 }
 
