@@ -91,3 +91,29 @@ def segments(parts, rows, device="cpu"):
     i32 = dict(dtype=torch.int32, device=device)
     return AttnMeta(positions=torch.tensor(pos, **i32), slots=None, block_tables=None, seq_lens=None,
                     q_start=torch.tensor(qs, **i32), state_rows=torch.tensor(rows, **i32), token_seq=torch.tensor(seg, **i32))
+
+
+def random_config(seed):
+    """A configuration drawn from a seed: sizes, head counts, layer order, windows, taps, constants."""
+    import random
+    r = random.Random(seed)
+    even = lambda lo, hi: 2 * r.randint(lo // 2, hi // 2)  # noqa: E731
+    layers = []
+    for _ in range(r.randint(2, 5)):
+        ff = r.choice([0, 24, 40, 72])
+        if r.random() < 0.55:
+            kv = r.choice([1, 2, 3])
+            heads = kv * r.choice([1, 2, 4])
+            dim, vdim = even(6, 80), even(6, 80)
+            rot = r.choice([0, even(2, dim), dim])
+            scaling = r.choice([None, (r.choice([2.0, 4.0, 8.0]), 1.0, r.choice([2.0, 4.0]), r.choice([16, 64, 256]))])
+            l = left(heads, kv, dim, vdim, r.choice([0, 2, 3, 4, 5]), r.choice([0, 1, 5, 16, 23, 64]), rot,
+                     r.choice([100.0, 10000.0, 500000.0]), scaling if rot else None, r.choice([None, 0.2, 0.05]))
+            layers.append(parallel(l, r.randint(1, 4), even(4, 72), r.randint(3, 72), ff))
+        else:
+            kv = r.choice([1, 2, 3])
+            layers.append(delta(kv * r.choice([1, 2]), kv, even(4, 100), r.randint(3, 72), r.choice([0, 2, 4]), ff,
+                                (r.randint(2, 9), r.randint(2, 9))))
+    return config(layers, width=even(24, 96), vocab=r.randint(20, 90),
+                  bigram=r.choice([None, (r.randint(5, 40), r.randint(1, 2000), r.randint(1, 50))]),
+                  scale=r.choice([1.0, 3.0]), eps=r.choice([1e-5, 1e-6]), mult=r.choice([1.0, 0.7, 0.4]))

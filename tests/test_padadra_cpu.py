@@ -381,3 +381,30 @@ def test_generate_command_line(tmp_path, capsys):
     for p, line in zip(prompts, lines):
         ids = [int(t) for t in line.split()]
         assert len(ids) == 3 and ids[0] == int(O.forward(sd, cfg, p)[-1].argmax())
+
+
+@pytest.mark.parametrize("seed", range(8, 13))
+def test_drawn_configurations(tmp_path, seed):
+    """Configurations drawn from a seed (sizes, head counts, layer order, windows, taps, constants):
+    a whole prompt against the same prompt in portions beside another request."""
+    cfg = C.random_config(seed)
+    path = str(tmp_path / "m")
+    sd = O.to_f64(C.checkpoint(cfg, path, seed=seed))
+    eng = C.engine(path, pool_tokens=256)
+    try:
+        a, b = C.tokens(60, cfg["vocab"], seed), C.tokens(23, cfg["vocab"], seed + 100)
+        wa, wb = O.forward(sd, cfg, a), O.forward(sd, cfg, b)
+        _close(eng.stream_step([("w", a, list(range(60)))], end=["w"]), wa)
+        at = 0
+        for i, s in enumerate([3, 2, 30, 1, 1, 17, 2, 4]):
+            entries, want = [("a", a[at:at + s], list(range(s)))], [wa[at:at + s]]
+            at += s
+            if i < 23:
+                entries.append(("b", b[i:i + 1], [0]))
+                want.append(wb[i:i + 1])
+            _close(eng.stream_step(entries), np.concatenate(want))
+        assert at == 60
+        eng.stream_step([("b", b[8:], [])], end=["a", "b"])
+        assert not any(eng.slots)
+    finally:
+        eng.shutdown()

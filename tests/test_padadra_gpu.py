@@ -114,3 +114,31 @@ def test_greedy_generation(tmp_path, graphs):
                 seq.append(tok)
     finally:
         eng.shutdown()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_drawn_configurations(tmp_path, seed):
+    """Configurations drawn from a seed (sizes, head counts, layer order, windows, taps, constants):
+    a whole prompt, the same prompt in portions and token by token, and two requests side by side."""
+    cfg = C.random_config(seed)
+    path = str(tmp_path / "m")
+    sd = O.to_f64(C.checkpoint(cfg, path, seed=seed))
+    eng = C.engine(path, backend="hip", dtype=torch.float32, pool_tokens=256)
+    try:
+        a, b = C.tokens(90, cfg["vocab"], seed), C.tokens(41, cfg["vocab"], seed + 100)
+        wa, wb = O.forward(sd, cfg, a), O.forward(sd, cfg, b)
+        _close(eng.stream_step([("w", a, list(range(90)))], end=["w"]), wa, "float32")
+        at, bt = 0, 0
+        for i, s in enumerate([3, 2, 30, 1, 1, 17, 2, 16, 1] + [1] * 17):
+            entries, want = [("a", a[at:at + s], list(range(s)))], [wa[at:at + s]]
+            at += s
+            if bt < 41:
+                n = min([1, 7, 2, 16][i % 4], 41 - bt)
+                entries.append(("b", b[bt:bt + n], list(range(n))))
+                want.append(wb[bt:bt + n])
+                bt += n
+            _close(eng.stream_step(entries, [k for k, done in (("a", at == 90), ("b", bt == 41 and n > 0)) if done and any(e[0] == k for e in entries)]),
+                   np.concatenate(want), "float32")
+        assert at == 90
+    finally:
+        eng.shutdown()

@@ -85,7 +85,7 @@ def test_short_conv_and_its_state(ops, dtype, taps, act, Cn, pad):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,d,e,rot", [(4, 2, 16, 24, 8), (2, 1, 24, 16, 24), (3, 3, 10, 12, 0), (6, 2, 72, 40, 36)])
+@pytest.mark.parametrize("H,G,d,e,rot", [(4, 2, 16, 24, 8), (2, 1, 24, 16, 24), (3, 3, 10, 12, 0), (6, 2, 72, 40, 36), (2, 2, 6, 10, 6)])
 def test_rope_pairs_kv_write_and_rotate_back(ops, dtype, H, G, d, e, rot):
     g = torch.Generator().manual_seed(H)
     T, BS = 37, 16
@@ -138,7 +138,7 @@ def _attention_inputs(H, G, d, e, lens, q_lens, dtype, seed, loud=None):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d,e", [(8, 1, 64, 64), (4, 2, 16, 24), (6, 2, 72, 40), (34, 2, 32, 32), (4, 2, 128, 128),
-                                     (2, 1, 64, 128), (3, 1, 96, 96)])
+                                     (2, 1, 64, 128), (3, 1, 96, 96), (2, 1, 18, 10)])
 @pytest.mark.parametrize("window", [0, 1, 16, 37, 96, 400])
 def test_window_and_sink_attention(ops, dtype, H, G, d, e, window):
     """Prefill tiles and single rows in one step; the loud key sits just outside the last query's
