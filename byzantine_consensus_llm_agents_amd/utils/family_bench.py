@@ -288,6 +288,15 @@ def state_kernels(s, dev):
         io = rows_ * (2 * Gq * 128 * 4 + H * 128 * 4 + H * 128 * 2 + H * 128 * 4) + (m_.q_start.numel() - 1) * H * 128 * 128 * 4 * 2
         out[f"state_scan_{name}"] = {"padadra_ms": round(t * 1e3, 4),
                                      "padadra_roof_frac": round(max(flops / PEAK_VALU, io / PEAK_BW) / t, 4)}
+    # ---- the recurrence: HGRN2, H / 2 heads of 64 x 128 state ----
+    Hh = max(1, H // 2)
+    q32, k32, g32 = (torch.rand(T, Hh, 64, device=dev) for _ in range(3))
+    v = torch.randn(T, Hh * 128, device=dev, dtype=bf)
+    S = torch.zeros(n + 1, Hh, 64, 128, device=dev)
+    t = _time(lambda: ops.gated_state_scan(q32, k32, g32, v, None, meta, S, False), iters=10)
+    io = T * (3 * Hh * 64 * 4 + Hh * 128 * 2 + Hh * 128 * 4)
+    out["state_scan_prefill_hgrn2"] = {"padadra_ms": round(t * 1e3, 4),
+                                       "padadra_roof_frac": round(max(T * Hh * 64 * 128 * 6 / PEAK_VALU, io / PEAK_BW) / t, 4)}
     return out
 
 

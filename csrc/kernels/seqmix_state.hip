@@ -19,7 +19,7 @@ namespace {
 
 constexpr int NT = 256;
 constexpr int MAX_TAPS = 16;
-constexpr int SCAN_CHUNK = 4;
+constexpr int SCAN_CHUNK_ELEMS = 512;   // rows x tokens of a recurrence staged through LDS at a time
 constexpr int SCAN_WAVES = 4;   // waves of a recurrence workgroup (8 value columns each)   // tokens of a recurrence staged through LDS at a time
 
 __device__ __forceinline__ float block_sum(float v, float* red) {
@@ -416,7 +416,7 @@ __global__ __launch_bounds__(NT) void delta_prepare_kernel(const T* __restrict__
 // columns: lane = 8 column + row group, so a lane keeps
 // dim / 8 rows of one column of S in registers and the two sums over rows (S^T k and S^T q) are
 // finished inside a group of 8 neighbouring lanes with three DPP adds (no LDS round trip).  The
-// tokens' q / k / g vectors are staged through LDS SCAN_CHUNK tokens at a time (every lane reads
+// tokens' q / k / g vectors are staged through LDS a few tokens at a time (every lane reads
 // its row group's 16-byte pieces; the groups' pieces are padded apart so that they fall into
 // different banks) by the whole workgroup, so a head's vectors are fetched once per 8 SCAN_WAVES
 // columns; the next chunk's loads fly under this chunk's arithmetic.
@@ -449,7 +449,7 @@ __global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a)
   constexpr int VP = 8 * GP;                         // one staged vector
   constexpr int NTH = 64 * SCAN_WAVES;
   constexpr int NL = (3 * DMAX + NTH - 1) / NTH;     // staged elements per thread and token: q | k | g
-  constexpr int CT = SCAN_CHUNK;                     // tokens staged at a time
+  constexpr int CT = SCAN_CHUNK_ELEMS / DMAX;        // tokens staged at a time: fewer, longer waits for narrow states
   __shared__ __attribute__((aligned(16))) float vec[2][CT][3 * VP];
   const int tid = threadIdx.x, lane = tid & 63, col = lane >> 3, rg = lane & 7;
   const int b = blockIdx.x, h = blockIdx.y, j = (blockIdx.z * SCAN_WAVES + (tid >> 6)) * 8 + col;
@@ -502,6 +502,7 @@ __global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a)
   for (int first = t0; first < t1; first += CT, buf ^= 1) {
     const bool more = first + CT < t1;
     if (more) load(first + CT, nxt);
+    float keep[(CT + 7) / 8];   // outputs of the chunk: the lane of row group r keeps tokens r, r + 8, ...
 #pragma unroll
     for (int tt = 0; tt < CT; ++tt) {
       const int t = first + tt;
@@ -536,13 +537,20 @@ __global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a)
             o[i] += S[4 * m + i] * q4[i];
           }
         }
-        const float os = group8_sum((o[0] + o[1]) + (o[2] + o[3]));
-        if (col_ok && rg == 0) a.out[(static_cast<size_t>(t) * a.H + h) * vdim + j] = os;
+        const float os = group8_sum((o[0] + o[1]) + (o[2] + o[3]));   // (in every lane of the group)
+        if (rg == (tt & 7)) keep[tt >> 3] = os;
       }
     }
     if (more) {
       stage(buf ^ 1, nxt);   // (the other buffer: its readers finished before the last barrier)
       cur = nxt;
+    }
+    // one store per 8 tokens, after the wait for the next chunk's loads: a store in flight never
+    // stands between a load and its use
+#pragma unroll
+    for (int r = 0; r < (CT + 7) / 8; ++r) {
+      const int t = first + 8 * r + rg;
+      if (col_ok && 8 * r + rg < CT && t < t1) a.out[(static_cast<size_t>(t) * a.H + h) * vdim + j] = keep[r];
     }
     __syncthreads();
   }
