@@ -142,3 +142,24 @@ def test_drawn_configurations(tmp_path, seed):
         assert at == 90
     finally:
         eng.shutdown()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_context_window_across_decode_splits(tmp_path, dtype):
+    """A window longer than a decode split and a context several windows long: the decode kernel
+    starts at the window's first split, the recurrences run hundreds of tokens."""
+    cfg = C.config([C.parallel(C.left(4, 2, 32, 32, 4, 200, 16, 50000.0, (4.0, 1.0, 4.0, 128)), 2, 16, 32, 48),
+                    C.delta(2, 2, 32, 16, 4, 48)], width=64, vocab=80)
+    path = str(tmp_path / "m")
+    sd = O.to_f64(C.checkpoint(cfg, path, seed=11))
+    eng = C.engine(path, backend="hip", dtype=getattr(torch, dtype), pool_tokens=1024, max_len=1024)
+    try:
+        toks = C.tokens(700, cfg["vocab"], 3)
+        want = O.forward(sd, cfg, toks)
+        idx = list(range(0, 520, 7)) + [519]
+        _close(eng.stream_step([("x", toks[:520], idx)]), want[idx], dtype)
+        got = [eng.stream_step([("x", toks[p:p + 1], [0])]) for p in range(520, 600)]
+        _close(torch.cat(got), want[520:600], dtype)
+        _close(eng.stream_step([("x", toks[600:], list(range(100)))], end=["x"]), want[600:], dtype)
+    finally:
+        eng.shutdown()
