@@ -214,6 +214,25 @@ def test_gated_state_scan(ops, dtype, H, Gq, d, e, delta):
     torch.testing.assert_close(sd.cpu(), state, atol=2e-4, rtol=2e-4)   # rows of segments moved on, row 5 untouched
 
 
+@pytest.mark.parametrize("d,delta", [(64, False), (128, True), (40, True)])
+def test_gated_state_scan_many_workgroups(ops, d, delta):
+    """Enough (segment, head, column) work that the kernel takes its 8-columns-per-wave form."""
+    g = torch.Generator().manual_seed(d)
+    H, Gq, e = 16, 8, 128
+    parts = [(0, 3), (5, 1), (2, 6), (0, 1), (9, 2), (1, 1), (0, 5), (3, 4)]
+    mc, md = _meta(parts, [1, 0, 3, 2, 5, 4, 7, 6])
+    T = mc.positions.numel()
+    q, k = torch.randn(T, Gq, d, generator=g) * 0.3, torch.randn(T, Gq, d, generator=g) * 0.3
+    gg, v = torch.rand(T, H, d, generator=g), torch.randn(T, H * e, generator=g).to(torch.bfloat16)
+    beta = torch.rand(T, H, generator=g) if delta else None
+    state = torch.randn(9, H, d, e, generator=g)
+    sd = state.to(DEV)
+    want = ref.gated_state_scan(q, k, gg, v, beta, mc, state, delta)
+    got = ops.gated_state_scan(q.to(DEV), k.to(DEV), gg.to(DEV), v.to(DEV), beta.to(DEV) if delta else None, md, sd, delta)
+    torch.testing.assert_close(got.cpu(), want, atol=2e-4, rtol=2e-4)
+    torch.testing.assert_close(sd.cpu(), state, atol=2e-4, rtol=2e-4)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_prepare_and_head_norm(ops, dtype):
     g = torch.Generator().manual_seed(3)
