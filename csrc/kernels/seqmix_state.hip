@@ -466,23 +466,41 @@ __global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a)
   for (int i = 0; i < RPL; ++i) S[i] = (load_state && rg * RPL + i < dim) ? Sp[static_cast<size_t>(i) * vdim] : 0.f;
   const T* vbase = static_cast<const T*>(a.v) + h * vdim + (col_ok ? j : 0);
 
-  // element e of a token is (which of q, k, g; row); rows past dim are zero
+  // element e of a token is (which of q, k, g; row); rows past dim are zero.  A thread's sources
+  // are walked token by token (chunks are loaded in order): one pointer step per element and
+  // token instead of the full address arithmetic
   struct Chunk { float r[CT][NL], v[CT], be[CT]; };
+  const float* src[NL];
+  int64_t step[NL];
+  bool src_ok[NL];
+#pragma unroll
+  for (int n = 0; n < NL; ++n) {
+    const int e = tid + NTH * n, which = e / DMAX, i = e - which * DMAX;
+    src_ok[n] = which < 3 && i < dim;
+    const float* p = which == 0 ? a.q + (static_cast<size_t>(t0) * a.Gq + gq) * dim
+                   : which == 1 ? a.k + (static_cast<size_t>(t0) * a.Gq + gq) * dim
+                                : a.g + (static_cast<size_t>(t0) * a.H + h) * dim;
+    src[n] = p + (src_ok[n] ? i : 0);
+    step[n] = which < 2 ? static_cast<int64_t>(a.Gq) * dim : static_cast<int64_t>(a.H) * dim;
+  }
+  const T* vsrc = vbase + static_cast<size_t>(t0) * a.v_stride;
+  const float* bsrc = DELTA ? a.beta + static_cast<size_t>(t0) * a.H + h : nullptr;
   auto load = [&](int first, Chunk& c) {
 #pragma unroll
     for (int tt = 0; tt < CT; ++tt) {
-      const int t = first + tt;
-      const bool live = t < t1;
+      const bool live = first + tt < t1;
 #pragma unroll
       for (int n = 0; n < NL; ++n) {
-        const int e = tid + NTH * n, which = e / DMAX, i = e - which * DMAX;
-        const float* p = which == 0 ? a.q + (static_cast<size_t>(t) * a.Gq + gq) * dim
-                       : which == 1 ? a.k + (static_cast<size_t>(t) * a.Gq + gq) * dim
-                                    : a.g + (static_cast<size_t>(t) * a.H + h) * dim;
-        c.r[tt][n] = (live && which < 3 && i < dim) ? p[i] : 0.f;
+        c.r[tt][n] = (live && src_ok[n]) ? *src[n] : 0.f;
+        src[n] += step[n];
       }
-      c.v[tt] = (live && col_ok) ? Elem<T>::ld(vbase[static_cast<size_t>(t) * a.v_stride]) : 0.f;
-      c.be[tt] = (DELTA && live) ? a.beta[static_cast<size_t>(t) * a.H + h] : 1.0f;
+      c.v[tt] = (live && col_ok) ? Elem<T>::ld(*vsrc) : 0.f;
+      vsrc += a.v_stride;
+      c.be[tt] = 1.0f;
+      if (DELTA) {
+        if (live) c.be[tt] = *bsrc;
+        bsrc += a.H;
+      }
     }
   };
   auto stage = [&](int buf, const Chunk& c) {
