@@ -172,7 +172,7 @@ def seqstate_ops(lib):
         Gq = q.shape[1]
         for t, name in ((q, "q"), (k, "k")):
             _req(t.dtype == torch.float32 and t.is_contiguous() and t.shape == (T, Gq, dim), f"{name} fp32 [T, Gq, dim]")
-        _req(g.dtype == torch.float32 and g.is_contiguous() and H % Gq == 0 and 1 <= dim <= 128, "g fp32 [T, H, dim], dim <= 128")
+        _req(g.dtype == torch.float32 and g.is_contiguous() and H % Gq == 0 and 1 <= dim <= 256, "g fp32 [T, H, dim], dim <= 256")
         _req(v.dim() == 2 and v.stride(1) == 1 and v.shape == (T, H * vdim), "v [T, H vdim], unit column stride")
         if delta:
             _req(beta is not None and beta.dtype == torch.float32 and beta.is_contiguous() and beta.shape == (T, H), "beta fp32 [T, H]")

@@ -606,7 +606,8 @@ int launch_scan(const ScanArgs& a, int B, hipStream_t s) {
   dim3 grid(B, a.H, (a.vdim + 8 * SCAN_WAVES - 1) / (8 * SCAN_WAVES));
   if (a.dim <= 32) state_scan_kernel<T, 32, DELTA><<<grid, 64 * SCAN_WAVES, 0, s>>>(a);
   else if (a.dim <= 64) state_scan_kernel<T, 64, DELTA><<<grid, 64 * SCAN_WAVES, 0, s>>>(a);
-  else state_scan_kernel<T, 128, DELTA><<<grid, 64 * SCAN_WAVES, 0, s>>>(a);
+  else if (a.dim <= 128) state_scan_kernel<T, 128, DELTA><<<grid, 64 * SCAN_WAVES, 0, s>>>(a);
+  else state_scan_kernel<T, 256, DELTA><<<grid, 64 * SCAN_WAVES, 0, s>>>(a);
   return BCG_CHECK_LAUNCH();
 }
 
@@ -754,7 +755,7 @@ BCG_API int bcg_gated_state_scan(const void* q32, const void* k32, const void* g
                                  void* state, int n_rows, void* out, int B, int H, int Gq, int dim, int vdim, int delta,
                                  int is_f32, void* stream) {
   if (B <= 0) return 0;
-  if (dim < 1 || dim > 128 || H <= 0 || Gq <= 0 || H % Gq || H > 65535 || (delta && beta == nullptr)) return -2;
+  if (dim < 1 || dim > 256 || H <= 0 || Gq <= 0 || H % Gq || H > 65535 || (delta && beta == nullptr)) return -2;
   ScanArgs a;
   a.q = static_cast<const float*>(q32); a.k = static_cast<const float*>(k32); a.g = static_cast<const float*>(g32);
   a.v = v; a.v_stride = v_stride; a.beta = static_cast<const float*>(beta);

@@ -197,7 +197,7 @@ def test_window_over_long_contexts(ops, window):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,Gq,d,e,delta", [(4, 4, 48, 64, False), (6, 6, 64, 32, True), (4, 2, 16, 12, True), (2, 1, 96, 72, True),
-                                            (3, 3, 20, 130, False), (2, 2, 128, 8, True)])
+                                            (3, 3, 20, 130, False), (2, 2, 128, 8, True), (2, 1, 160, 24, True), (1, 1, 256, 40, False)])
 def test_gated_state_scan(ops, dtype, H, Gq, d, e, delta):
     g = torch.Generator().manual_seed(H * d)
     mc, md = _meta(PARTS, ROWS)
