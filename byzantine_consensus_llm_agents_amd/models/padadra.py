@@ -34,6 +34,9 @@ Kernel plan of one layer (HIP backend; the torch backend runs the same ops from
     residual_mix_norm          x += m (...) fused with the out-norms of both mixers and the NEXT
                                layer's two scalar norms
 
+Large prefill steps run the recurrent branch (prepare, scan, head norm) on a second stream
+beside the attention branch and the feed-forward.
+
 No host synchronisation anywhere: a decode step is capturable in a HIP graph.
 """
 
@@ -51,6 +54,10 @@ class PadadraModel:
     logits_dtype = torch.float32
     supports_cascade = False
     has_seq_state = True      # recurrent state: a cached prompt prefix cannot stand in for its tokens
+    # Packed steps of at least this many rows run a layer's recurrence on a second stream beside the
+    # attention branch and the feed-forward (the token-sequential scan leaves most of the chip idle);
+    # None = never.  Decode steps (captured into graphs) and small steps stay on one stream.
+    overlap_min_rows = 2048
 
     def __init__(self, cfg: PadadraConfig, ops, device, dtype=torch.bfloat16, tp: Optional[TPGroup] = None,
                  quant: Optional[str] = None):
@@ -63,6 +70,7 @@ class PadadraModel:
         self.layers: List[Dict[str, torch.Tensor]] = []
         self.embed = self.bigram = self.lm_head = None
         self.final_gain = 1.0
+        self._side_stream = None
         attn = [l.attn for l in cfg.layers if l.attn is not None]
         self.n_q = max([a.heads for a in attn] + [l.state.heads for l in cfg.layers])
         self.n_kv = max([a.kv_heads for a in attn] or [1])
@@ -255,6 +263,27 @@ class PadadraModel:
         L = self.layers[i]
         return (L["gain1"],) if L["gain2"] is None else (L["gain1"], L["gain2"])
 
+    def _fork(self, enabled: bool, fn):
+        """Queue ``fn()`` behind everything queued so far: on the side stream when ``enabled`` (the
+        caller goes on with independent work and calls the returned ``join`` before it reads the
+        result), else at once.  Returns ``join``: ``join()`` gives ``fn``'s result."""
+        if not enabled:
+            out = fn()
+            return lambda: out
+        main = torch.cuda.current_stream()
+        if self._side_stream is None:
+            self._side_stream = torch.cuda.Stream(self.device)
+        side = self._side_stream
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            out = fn()
+
+        def join():
+            main.wait_stream(side)
+            out.record_stream(main)   # allocated on the side stream, read on this one
+            return out
+        return join
+
     def forward(self, tokens: torch.Tensor, meta: AttnMeta, k_cache, v_cache, trace: Optional[list] = None):
         """Logits (fp32) of the rows ``meta.logits_idx`` (all rows when None).  ``meta.state`` holds
         the tables of `alloc_state`, ``meta.state_rows`` every segment's row in them.  ``trace``: a
@@ -268,29 +297,49 @@ class PadadraModel:
                                              c.bigram[1:] if c.bigram else None, eps, self._gains(0), dt)
         n_layers = len(c.layers)
         pos = meta.positions
+        overlap = (self.overlap_min_rows is not None and not meta.decode and tokens.numel() >= self.overlap_min_rows
+                   and self.device.type == "cuda" and not torch.cuda.is_current_stream_capturing())
         for i, (spec, L) in enumerate(zip(c.layers, self.layers)):
             s, S = spec.state, st["layers"][i]
             last = i == n_layers - 1
             sel = meta.logits_idx if last else None
             y = ops.linear(hs[0], L["fused"], L["bias"])
             normed, plain = [], []
+
+            def feed_forward():
+                """The layer's feed-forward (of the rows still needed); independent of the mixer."""
+                nonlocal x, hs
+                if sel is not None:
+                    x = x.index_select(0, sel)
+                    hs = tuple(h.index_select(0, sel) for h in hs)
+                if spec.mlp is not None:
+                    plain.append(ops.linear(ops.act_fn(ops.linear(hs[1], L["up"]), "relu2"), L["down"]))
+
             if spec.attn is not None:
                 a = spec.attn
                 cw = a.q_width + a.k_width + a.v_width
+                n = s.heads * s.dim
+
+                def recurrent_branch():
+                    q32, k32, g32 = ops.hgrn2_prepare(y, cw, cw + n, s.heads, s.dim, L["f_bias"], L["lower"])
+                    o32 = ops.gated_state_scan(q32, k32, g32, y[:, cw + 2 * n:cw + 2 * n + s.heads * s.vdim], None, meta,
+                                               S["S"], False)
+                    if sel is not None:
+                        o32 = o32.index_select(0, sel)
+                    return ops.head_norm_gate(o32, L["head_norm"], eps, None, dt)
+
+                join = self._fork(overlap, recurrent_branch)
                 u = ops.short_conv(y, cw, L["conv_w"], meta, S["conv"]) if a.conv else y
                 q = ops.rope_pairs_kv_write(u, pos, meta.slots, a.heads, a.kv_heads, a.dim, a.vdim, L["q_norm"], L["k_norm"],
                                             eps, L["inv_freq"], L["v_inv_freq"], k_cache[i], v_cache[i])
                 att = ops.multimap_attention(q, k_cache[i], v_cache[i], meta, a.scale, 1, 0.0, -1.0, 1.0, a.vdim,
                                              a.window, L["sink"])
-                n = s.heads * s.dim
-                q32, k32, g32 = ops.hgrn2_prepare(y, cw, cw + n, s.heads, s.dim, L["f_bias"], L["lower"])
-                o32 = ops.gated_state_scan(q32, k32, g32, y[:, cw + 2 * n:cw + 2 * n + s.heads * s.vdim], None, meta,
-                                           S["S"], False)
                 if sel is not None:
-                    att, o32, pos = att.index_select(0, sel), o32.index_select(0, sel), pos.index_select(0, sel)
+                    att, pos = att.index_select(0, sel), pos.index_select(0, sel)
                 att = ops.rotate_pairs(att, pos, L["v_inv_freq"], -1.0, a.heads)
-                r = ops.head_norm_gate(o32, L["head_norm"], eps, None, dt)
-                normed = [(ops.linear(att, L["o_left"]), L["out_left"]), (ops.linear(r, L["o_right"]), L["out_right"])]
+                normed = [(ops.linear(att, L["o_left"]), L["out_left"])]
+                feed_forward()
+                normed.append((ops.linear(join(), L["o_right"]), L["out_right"]))
             else:
                 nqk = s.kv_heads * s.dim
                 cw = 2 * nqk + s.heads * s.vdim
@@ -299,17 +348,18 @@ class PadadraModel:
                 off_g = off_a + L["rank_a"]
                 decay = ops.linear(y[:, off_a:off_g].contiguous(), L["a2"])
                 q32, k32, g32, beta = ops.delta_prepare(u, y, cw, decay, L["a_log"], L["dt_bias"], s.heads, s.kv_heads, s.dim)
-                o32 = ops.gated_state_scan(q32, k32, g32, u[:, 2 * nqk:], beta, meta, S["S"], True)
+
+                def recurrent_branch():
+                    o32 = ops.gated_state_scan(q32, k32, g32, u[:, 2 * nqk:], beta, meta, S["S"], True)
+                    return o32 if sel is None else o32.index_select(0, sel)
+
+                join = self._fork(overlap, recurrent_branch)
                 gate_in = y[:, off_g:off_g + L["rank_g"]]
                 if sel is not None:
-                    o32, gate_in = o32.index_select(0, sel), gate_in.index_select(0, sel)
+                    gate_in = gate_in.index_select(0, sel)
                 gate = ops.linear(gate_in.contiguous(), L["g2"])
-                plain = [ops.linear(ops.head_norm_gate(o32, L["head_norm"], eps, gate, dt), L["o"])]
-            if sel is not None:
-                x = x.index_select(0, sel)
-                hs = tuple(h.index_select(0, sel) for h in hs)
-            if spec.mlp is not None:
-                plain.append(ops.linear(ops.act_fn(ops.linear(hs[1], L["up"]), "relu2"), L["down"]))
+                feed_forward()
+                plain.insert(0, ops.linear(ops.head_norm_gate(join(), L["head_norm"], eps, gate, dt), L["o"]))
             hs = ops.residual_mix_norm(x, normed, 0.5, plain, mult, eps, self._gains(i + 1), dt)
             if trace is not None:
                 trace.append(x.clone())

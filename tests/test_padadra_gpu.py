@@ -163,3 +163,25 @@ def test_long_context_window_across_decode_splits(tmp_path, dtype):
         _close(eng.stream_step([("x", toks[600:], list(range(100)))], end=["x"]), want[600:], dtype)
     finally:
         eng.shutdown()
+
+
+@pytest.mark.parametrize("name", list(C.CASES))
+def test_recurrent_branch_on_the_second_stream(tmp_path, name):
+    """Large prefill steps run the recurrence beside the attention branch and the feed-forward on
+    a second stream; here every step does, several times over, against the one-stream result."""
+    cfg = C.CASES[name]
+    path = str(tmp_path / "m")
+    sd = O.to_f64(C.checkpoint(cfg, path, seed=9))
+    eng = C.engine(path, backend="hip", dtype=torch.float32, pool_tokens=1024)
+    try:
+        eng.model.overlap_min_rows = 1
+        toks = [C.tokens(n, cfg["vocab"], 30 + n) for n in (200, 77, 130)]
+        want = [O.forward(sd, cfg, t) for t in toks]
+        for rep in range(4):
+            got = eng.stream_step([(f"s{i}", t[:50], list(range(50))) for i, t in enumerate(toks)])
+            _close(got, np.concatenate([w[:50] for w in want]), "float32")
+            got = eng.stream_step([(f"s{i}", t[50:], list(range(len(t) - 50))) for i, t in enumerate(toks)],
+                                  end=[f"s{i}" for i in range(3)])
+            _close(got, np.concatenate([w[50:] for w in want]), "float32")
+    finally:
+        eng.shutdown()
