@@ -116,18 +116,19 @@ def test_greedy_generation(tmp_path, graphs):
         eng.shutdown()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("seed", range(8))
-def test_drawn_configurations(tmp_path, seed):
+def test_drawn_configurations(tmp_path, seed, dtype):
     """Configurations drawn from a seed (sizes, head counts, layer order, windows, taps, constants):
     a whole prompt, the same prompt in portions and token by token, and two requests side by side."""
     cfg = C.random_config(seed)
     path = str(tmp_path / "m")
     sd = O.to_f64(C.checkpoint(cfg, path, seed=seed))
-    eng = C.engine(path, backend="hip", dtype=torch.float32, pool_tokens=256)
+    eng = C.engine(path, backend="hip", dtype=getattr(torch, dtype), pool_tokens=256)
     try:
         a, b = C.tokens(90, cfg["vocab"], seed), C.tokens(41, cfg["vocab"], seed + 100)
         wa, wb = O.forward(sd, cfg, a), O.forward(sd, cfg, b)
-        _close(eng.stream_step([("w", a, list(range(90)))], end=["w"]), wa, "float32")
+        _close(eng.stream_step([("w", a, list(range(90)))], end=["w"]), wa, dtype)
         at, bt = 0, 0
         for i, s in enumerate([3, 2, 30, 1, 1, 17, 2, 16, 1] + [1] * 17):
             entries, want = [("a", a[at:at + s], list(range(s)))], [wa[at:at + s]]
@@ -138,7 +139,7 @@ def test_drawn_configurations(tmp_path, seed):
                 want.append(wb[bt:bt + n])
                 bt += n
             _close(eng.stream_step(entries, [k for k, done in (("a", at == 90), ("b", bt == 41 and n > 0)) if done and any(e[0] == k for e in entries)]),
-                   np.concatenate(want), "float32")
+                   np.concatenate(want), dtype)
         assert at == 90
     finally:
         eng.shutdown()
